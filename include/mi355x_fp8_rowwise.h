@@ -1,0 +1,108 @@
+/*
+ * mi355x_fp8_rowwise.h -- C ABI of the MI355X (gfx950 / CDNA4) row-wise scaled FP8 GEMM library.
+ *
+ * The library stands in for the native kernels the tritonbench operator
+ * `fp8_gemm_rowwise` reaches through FBGEMM:
+ *   - tritonbench/operators/fp8_gemm_rowwise/operator.py:187-199
+ *       matmul_fp8_row(xq, wq, x_scale, w_scale, bias=...)          (fused bias)
+ *   - tritonbench/operators/fp8_gemm_rowwise/operator.py:201-217
+ *       torch.ops.fbgemm.f8f8bf16_rowwise(xq, wq, x_scale, w_scale) (baseline backend)
+ *   - tritonbench/operators/fp8_gemm_rowwise/operator.py:136-145
+ *       fp8_row_quantize(x)                                         (input preparation)
+ * The reference defines no C interface of its own for this path (FBGEMM is reached
+ * through torch.ops / Python); the entry points below are what a ctypes / pybind
+ * binding on the reference side would call.
+ *
+ * Conventions
+ *   - every data pointer is a DEVICE pointer on the current HIP device;
+ *   - matrices are row-major, leading dimensions are in ELEMENTS;
+ *   - fp8 is OCP e4m3fn (bias 7, max 448, no inf, NaN = 0x7f/0xff), one byte per element;
+ *   - bf16 is the upper 16 bits of an IEEE binary32, rounded to nearest even;
+ *   - `stream` is a hipStream_t passed as void* (NULL = the null stream);
+ *   - calls only ENQUEUE work: no allocation, no host synchronisation, so they may be
+ *     recorded into a HIP graph;
+ *   - the library borrows all pointers for the duration of the enqueued work and owns
+ *     no device memory.
+ *
+ * Status codes: 0 ok, MI355X_FP8_EINVAL bad argument, MI355X_FP8_ENOTSUP shape or
+ * alignment outside what the kernels handle, MI355X_FP8_ELAUNCH the HIP runtime
+ * reported an error at launch. mi355x_fp8_rowwise_last_error() returns a
+ * thread-local, NUL-terminated description of the last non-zero status.
+ */
+#ifndef MI355X_FP8_ROWWISE_H
+#define MI355X_FP8_ROWWISE_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define MI355X_FP8_ABI_VERSION 1
+
+#define MI355X_FP8_OK        0
+#define MI355X_FP8_EINVAL   (-1)
+#define MI355X_FP8_ENOTSUP  (-2)
+#define MI355X_FP8_ELAUNCH  (-3)
+
+/* Kernel families. AUTO lets the library pick from (M, N, K). */
+#define MI355X_FP8_VARIANT_AUTO    0
+#define MI355X_FP8_VARIANT_TILED   1  /* LDS-tiled persistent MFMA kernel (compute-bound shapes) */
+#define MI355X_FP8_VARIANT_SKINNY  2  /* in-workgroup split-K streaming kernel (M <= 64, HBM-bound) */
+
+/* Source element types accepted by the quantiser. */
+#define MI355X_FP8_SRC_F32   0
+#define MI355X_FP8_SRC_BF16  1
+
+int mi355x_fp8_rowwise_abi_version(void);
+
+const char* mi355x_fp8_rowwise_last_error(void);
+
+/* Variant AUTO would run for this shape (one of the MI355X_FP8_VARIANT_* values > 0),
+ * or a negative status when the shape is not supported. Lets tests pin the dispatch. */
+int mi355x_fp8_rowwise_select_variant(int64_t M, int64_t N, int64_t K);
+
+/* Bytes of device workspace `variant` needs for this shape (0 when none). */
+size_t mi355x_fp8_rowwise_workspace_bytes(int64_t M, int64_t N, int64_t K, int variant);
+
+/*
+ * C[M,N] (bf16) = bf16( (sum_k A[m,k] * B[n,k]) * a_scale[m] * b_scale[n] + bias[n] )
+ *
+ * Replaces the timed callables of operator.py:187-199 (bias fused before the single
+ * bf16 rounding, as matmul_fp8_row does) and operator.py:201-217.
+ *
+ *   a        e4m3fn [M, K], row stride lda      b        e4m3fn [N, K], row stride ldb
+ *   a_scale  f32 [M]                            b_scale  f32 [N]
+ *   bias     bf16 [N] or NULL                   c        bf16 [M, N], row stride ldc
+ *
+ * Requirements: M, N, K >= 1; K, lda, ldb multiples of 16; a and b 16-byte aligned.
+ * `workspace` may be NULL when mi355x_fp8_rowwise_workspace_bytes() is 0.
+ */
+int mi355x_fp8_rowwise_gemm(const void* a, const void* b,
+                            const float* a_scale, const float* b_scale,
+                            const void* bias, void* c,
+                            int64_t M, int64_t N, int64_t K,
+                            int64_t lda, int64_t ldb, int64_t ldc,
+                            void* workspace, size_t workspace_bytes,
+                            int variant, void* stream);
+
+/*
+ * Row-wise e4m3fn quantiser, replacing fp8_row_quantize (operator.py:136-145):
+ *   amax[r]      = max_k |x[r,k]|
+ *   scale[r]     = 448 / max(amax[r], 1e-12)
+ *   xq[r,k]      = e4m3fn( clamp(x[r,k] * scale[r], -448, 448) )     (round to nearest even)
+ *   inv_scale[r] = 1 / scale[r]                                      (f32)
+ * The arithmetic runs in f32 (a bf16 source is widened first).
+ *
+ *   x  [R, K] of `src_type`, row stride ldx (elements)     xq  e4m3fn [R, K], row stride ldq
+ */
+int mi355x_fp8_rowwise_quantize(const void* x, int src_type,
+                                void* xq, float* inv_scale,
+                                int64_t R, int64_t K, int64_t ldx, int64_t ldq,
+                                void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* MI355X_FP8_ROWWISE_H */

@@ -1,0 +1,98 @@
+"""ctypes binding of the C ABI declared in include/mi355x_fp8_rowwise.h.
+
+The shared library is loaded from tritonbench_amd/lib/ (built in-tree by
+tritonbench_amd.build). There is no fallback: if the library is missing or does not
+load, every entry point raises.
+"""
+import ctypes
+import os
+import threading
+from ctypes import c_char_p, c_int, c_int64, c_size_t, c_void_p
+
+from .build import LIB_PATH
+
+ABI_VERSION = 1
+
+OK = 0
+EINVAL = -1
+ENOTSUP = -2
+ELAUNCH = -3
+
+VARIANT_AUTO = 0
+VARIANT_TILED = 1
+VARIANT_SKINNY = 2
+
+SRC_F32 = 0
+SRC_BF16 = 1
+
+# symbol -> (restype, argtypes); must list every function the header declares
+SIGNATURES = {
+    "mi355x_fp8_rowwise_abi_version": (c_int, []),
+    "mi355x_fp8_rowwise_last_error": (c_char_p, []),
+    "mi355x_fp8_rowwise_select_variant": (c_int, [c_int64, c_int64, c_int64]),
+    "mi355x_fp8_rowwise_workspace_bytes": (c_size_t, [c_int64, c_int64, c_int64, c_int]),
+    "mi355x_fp8_rowwise_gemm": (
+        c_int,
+        [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
+         c_int64, c_int64, c_int64, c_int64, c_int64, c_int64,
+         c_void_p, c_size_t, c_int, c_void_p],
+    ),
+    "mi355x_fp8_rowwise_quantize": (
+        c_int,
+        [c_void_p, c_int, c_void_p, c_void_p, c_int64, c_int64, c_int64, c_int64, c_void_p],
+    ),
+}
+
+_lock = threading.Lock()
+_lib = None
+
+
+class LibraryNotBuilt(RuntimeError):
+    pass
+
+
+def library_path() -> str:
+    return LIB_PATH
+
+
+def load() -> ctypes.CDLL:
+    """Loads the library once and checks its ABI version."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    with _lock:
+        if _lib is not None:
+            return _lib
+        if not os.path.exists(LIB_PATH):
+            raise LibraryNotBuilt(
+                f"{LIB_PATH} does not exist; build it with `python -m tritonbench_amd.build` "
+                "(needs hipcc). There is no CPU or PyTorch fallback for this operator."
+            )
+        lib = ctypes.CDLL(LIB_PATH)
+        for name, (restype, argtypes) in SIGNATURES.items():
+            fn = getattr(lib, name)  # AttributeError if the symbol is missing
+            fn.restype = restype
+            fn.argtypes = argtypes
+        got = lib.mi355x_fp8_rowwise_abi_version()
+        if got != ABI_VERSION:
+            raise RuntimeError(f"{LIB_PATH}: ABI version {got}, this binding expects {ABI_VERSION}")
+        _lib = lib
+    return _lib
+
+
+def last_error() -> str:
+    msg = load().mi355x_fp8_rowwise_last_error()
+    return msg.decode("utf-8", "replace") if msg else ""
+
+
+def check(status: int, what: str) -> None:
+    """Maps a C status to the exception the benchmark harness understands:
+    NotImplementedError becomes a "not supported" cell, anything else propagates."""
+    if status == OK:
+        return
+    msg = f"{what}: {last_error()} (status {status})"
+    if status == ENOTSUP:
+        raise NotImplementedError(msg)
+    if status == EINVAL:
+        raise ValueError(msg)
+    raise RuntimeError(msg)

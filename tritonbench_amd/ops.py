@@ -1,0 +1,110 @@
+"""PyTorch-facing wrappers around the C ABI. PyTorch supplies device memory and the
+current stream; all arithmetic happens in the HIP library."""
+from typing import Optional, Tuple
+
+import torch
+
+from . import _lib
+
+FP8_DTYPE = torch.float8_e4m3fn
+E4M3_MAX_POS = 448.0
+
+
+def _require_gpu(t: torch.Tensor, name: str) -> None:
+    if not t.is_cuda:
+        raise RuntimeError(
+            f"{name} is on {t.device}: the MI355X backend only runs on a ROCm device "
+            "(there is no CPU fallback)"
+        )
+
+
+def _stream_ptr() -> int:
+    return torch.cuda.current_stream().cuda_stream
+
+
+def select_variant(m: int, n: int, k: int) -> int:
+    v = _lib.load().mi355x_fp8_rowwise_select_variant(m, n, k)
+    if v < 0:
+        _lib.check(v, "select_variant")
+    return v
+
+
+def fp8_gemm_rowwise(
+    xq: torch.Tensor,
+    wq: torch.Tensor,
+    x_scale: torch.Tensor,
+    w_scale: torch.Tensor,
+    bias: Optional[torch.Tensor] = None,
+    out: Optional[torch.Tensor] = None,
+    variant: int = _lib.VARIANT_AUTO,
+) -> torch.Tensor:
+    """bf16 [M,N] = ((xq @ wq.T) * x_scale[:,None] * w_scale[None,:] + bias).
+
+    Same operands as the callables of tritonbench/operators/fp8_gemm_rowwise/operator.py:187-217:
+    xq [M,K] and wq [N,K] float8_e4m3fn, x_scale [M] and w_scale [N] float32, bias [N]
+    bfloat16 or None. Only enqueues work on the current stream (graph-capturable).
+    """
+    lib = _lib.load()
+    for t, name in ((xq, "xq"), (wq, "wq"), (x_scale, "x_scale"), (w_scale, "w_scale")):
+        _require_gpu(t, name)
+    if xq.dtype != FP8_DTYPE or wq.dtype != FP8_DTYPE:
+        raise TypeError(f"xq and wq must be {FP8_DTYPE}, got {xq.dtype} and {wq.dtype}")
+    if xq.dim() != 2 or wq.dim() != 2 or xq.shape[1] != wq.shape[1]:
+        raise ValueError(f"expected xq [M,K] and wq [N,K], got {tuple(xq.shape)} and {tuple(wq.shape)}")
+    m, k = xq.shape
+    n = wq.shape[0]
+    if x_scale.dtype != torch.float32 or w_scale.dtype != torch.float32:
+        raise TypeError("x_scale and w_scale must be float32")
+    if x_scale.numel() != m or w_scale.numel() != n:
+        raise ValueError("x_scale must have M entries and w_scale N entries")
+    if xq.stride(1) != 1 or wq.stride(1) != 1:
+        raise ValueError("xq and wq must be K-contiguous")
+    if not x_scale.is_contiguous() or not w_scale.is_contiguous():
+        raise ValueError("scales must be contiguous")
+    bias_ptr = None
+    if bias is not None:
+        _require_gpu(bias, "bias")
+        if bias.dtype != torch.bfloat16 or bias.numel() != n or not bias.is_contiguous():
+            raise ValueError("bias must be a contiguous bfloat16 vector of N entries")
+        bias_ptr = bias.data_ptr()
+    if out is None:
+        out = torch.empty((m, n), dtype=torch.bfloat16, device=xq.device)
+    else:
+        _require_gpu(out, "out")
+        if out.dtype != torch.bfloat16 or tuple(out.shape) != (m, n) or out.stride(1) != 1:
+            raise ValueError("out must be bfloat16 [M,N] with unit column stride")
+    ws_bytes = lib.mi355x_fp8_rowwise_workspace_bytes(m, n, k, variant)
+    ws = None
+    if ws_bytes:
+        ws = torch.empty(ws_bytes, dtype=torch.uint8, device=xq.device)
+    st = lib.mi355x_fp8_rowwise_gemm(
+        xq.data_ptr(), wq.data_ptr(), x_scale.data_ptr(), w_scale.data_ptr(), bias_ptr,
+        out.data_ptr(), m, n, k, xq.stride(0), wq.stride(0), out.stride(0),
+        ws.data_ptr() if ws is not None else None, ws_bytes, variant, _stream_ptr(),
+    )
+    _lib.check(st, "mi355x_fp8_rowwise_gemm")
+    return out
+
+
+def fp8_row_quantize(x: torch.Tensor) -> Tuple[torch.Tensor, torch.Tensor]:
+    """Row-wise e4m3fn quantisation on the GPU; returns (xq, inverse scale) like
+    fp8_row_quantize in tritonbench/operators/fp8_gemm_rowwise/operator.py:136-145."""
+    lib = _lib.load()
+    _require_gpu(x, "x")
+    if x.dim() != 2 or x.stride(1) != 1:
+        raise ValueError("x must be 2-D with unit column stride")
+    if x.dtype == torch.float32:
+        src = _lib.SRC_F32
+    elif x.dtype == torch.bfloat16:
+        src = _lib.SRC_BF16
+    else:
+        raise TypeError(f"unsupported source dtype {x.dtype}")
+    r, k = x.shape
+    xq = torch.empty((r, k), dtype=FP8_DTYPE, device=x.device)
+    inv_scale = torch.empty((r,), dtype=torch.float32, device=x.device)
+    st = lib.mi355x_fp8_rowwise_quantize(
+        x.data_ptr(), src, xq.data_ptr(), inv_scale.data_ptr(), r, k, x.stride(0), xq.stride(0),
+        _stream_ptr(),
+    )
+    _lib.check(st, "mi355x_fp8_rowwise_quantize")
+    return xq, inv_scale
