@@ -1,0 +1,226 @@
+"""Benchmark of the row-wise FP8 GEMM hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--all-configs] [--no-cpu-baseline]
+
+One step = one pass of the hot path (one mi355x_fp8_rowwise_gemm call through the C ABI)
+over the headline workload M=N=K=8192 with operands resident in HBM. Prints ONE JSON line:
+the headline TFLOP/s, the roofline of the dominant kernel measured with HIP events on the
+launch stream, the CPU baseline (the oracle's fp32 dequantise + torch.matmul, timed on this
+machine's host cores), and per-configuration figures for the skinny (HBM-bound) and the
+other benchmark shapes under "configs".
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+import torch
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+PEAK_FP8_TFLOPS = 5000.0  # dense FP8 MFMA, MI355X datasheet
+PEAK_HBM_GBPS = 8000.0    # HBM3E, MI355X datasheet
+SEED = 1337
+
+
+def make_device_inputs(m, n, k, sigma, bias, dev, copies=1):
+    """Seeded synthetic operands generated and quantised on the device (the HIP quantiser is
+    bit-exact against the oracle). `copies` > 1 returns independent operand sets to rotate
+    through so that no call finds its operands in L2 or the 256 MB memory-side cache."""
+    from tritonbench_amd import ops
+
+    g = torch.Generator(device=dev)
+    g.manual_seed(SEED + m * 7 + n * 3 + k)
+    sets = []
+    for _ in range(copies):
+        x = torch.randn((m, k), generator=g, device=dev, dtype=torch.float32) * sigma
+        w = torch.randn((n, k), generator=g, device=dev, dtype=torch.float32) * sigma
+        xq, xs = ops.fp8_row_quantize(x)
+        wq, ws = ops.fp8_row_quantize(w)
+        del x, w
+        b = (0.1 * torch.randn((n,), generator=g, device=dev, dtype=torch.float32)).to(torch.bfloat16) if bias else None
+        out = torch.empty((m, n), dtype=torch.bfloat16, device=dev)
+        sets.append((xq, wq, xs, ws, b, out))
+    return sets
+
+
+def time_steps(sets, steps, warmup):
+    """Average ms per call over exactly `steps` calls, HIP events on the launch stream."""
+    from tritonbench_amd import ops
+
+    stream = torch.cuda.current_stream()
+    for i in range(warmup):
+        xq, wq, xs, ws, b, out = sets[i % len(sets)]
+        ops.fp8_gemm_rowwise(xq, wq, xs, ws, bias=b, out=out)
+    torch.cuda.synchronize()
+    start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    start.record(stream)
+    for i in range(steps):
+        xq, wq, xs, ws, b, out = sets[i % len(sets)]
+        ops.fp8_gemm_rowwise(xq, wq, xs, ws, bias=b, out=out)
+    end.record(stream)
+    torch.cuda.synchronize()
+    return start.elapsed_time(end) / steps
+
+
+def time_steps_graph(sets, steps, warmup):
+    """Same, with the `steps` calls captured in one HIP graph (no per-launch host gaps);
+    this is how the benchmark harness times the operator."""
+    from tritonbench_amd import ops
+
+    side = torch.cuda.Stream()
+    with torch.cuda.stream(side):
+        for i in range(max(warmup, 1)):
+            xq, wq, xs, ws, b, out = sets[i % len(sets)]
+            ops.fp8_gemm_rowwise(xq, wq, xs, ws, bias=b, out=out)
+        torch.cuda.synchronize()
+        g = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g, stream=side):
+            for i in range(steps):
+                xq, wq, xs, ws, b, out = sets[i % len(sets)]
+                ops.fp8_gemm_rowwise(xq, wq, xs, ws, bias=b, out=out)
+        torch.cuda.synchronize()
+        best = None
+        for _ in range(3):
+            start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            start.record(side)
+            g.replay()
+            end.record(side)
+            torch.cuda.synchronize()
+            ms = start.elapsed_time(end) / steps
+            best = ms if best is None else min(best, ms)
+    return best
+
+
+def figures(m, n, k, bias, ms):
+    flops = 2 * m * n * k + (2 * m * n if bias else 0)
+    nbytes = m * k + n * k + 2 * m * n
+    tflops = flops / ms / 1e9
+    gbps = nbytes / ms / 1e6
+    t_mfma = flops / (PEAK_FP8_TFLOPS * 1e12)
+    t_hbm = nbytes / (PEAK_HBM_GBPS * 1e9)
+    bound = "mfma" if t_mfma >= t_hbm else "hbm"
+    frac = tflops / PEAK_FP8_TFLOPS if bound == "mfma" else gbps / PEAK_HBM_GBPS
+    return dict(us=ms * 1e3, tflops=tflops, gbps=gbps, bound=bound, frac=frac)
+
+
+def cpu_baseline(xq, wq, xs, ws, budget_s=12.0):
+    """The oracle (fp32 dequantise + torch.matmul) on host cores, on the same operands."""
+    from oracle import fp8_rowwise as orc
+
+    hxq, hwq, hxs, hws = xq.cpu(), wq.cpu(), xs.cpu(), ws.cpu()
+    m, k = hxq.shape
+    n = hwq.shape[0]
+    t0 = time.perf_counter()
+    orc.dequant_matmul(hxq, hwq, hxs, hws)  # warm-up (also pages in the BLAS)
+    first = time.perf_counter() - t0
+    times = []
+    spent = 0.0
+    while spent < budget_s and len(times) < 5:
+        t0 = time.perf_counter()
+        orc.dequant_matmul(hxq, hwq, hxs, hws)
+        dt = time.perf_counter() - t0
+        times.append(dt)
+        spent += dt
+    best = min(times) if times else first
+    return {
+        "value": 2 * m * n * k / best / 1e12,
+        "unit": "TFLOP/s",
+        "cores": torch.get_num_threads(),
+        "kind": "port",
+        "sample": f"full M=N=K=8192 workload, best of {len(times)} calls after 1 warm-up ({best:.3f} s/call, "
+                  f"dequantise included, host cpu_count {os.cpu_count()})",
+    }
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--all-configs", action="store_true", help="also time every Llama-3-70B projection shape")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-extra", action="store_true", help="headline workload only")
+    args = ap.parse_args()
+    if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        print("bench.py measures one GPU: this hot path is a single-device kernel and nothing here "
+              "uses a second GPU; run with --gpus 1", file=sys.stderr)
+        sys.exit(2)
+    if not torch.cuda.is_available():
+        print("bench.py needs a ROCm GPU (the HIP path has no CPU fallback)", file=sys.stderr)
+        sys.exit(2)
+    from tritonbench_amd import _lib
+
+    _lib.load()
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+
+    m = n = k = 8192
+    sets = make_device_inputs(m, n, k, 1.0, False, dev, copies=1)
+    torch.cuda.synchronize()
+    ms = time_steps(sets, args.steps, args.warmup)
+    head = figures(m, n, k, False, ms)
+
+    line = {
+        "metric": "fp8_gemm_rowwise TFLOP/s at M=N=K=8192 (1 GPU)",
+        "value": head["tflops"],
+        "unit": "TFLOP/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": ms,
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "fp8_e4m3fn x fp8_e4m3fn -> f32 accumulate -> bf16",
+        "data": "synthetic (seeded N(0,1) fp32, row-wise e4m3fn quantised on device)",
+        "config": {"workload": "c2_square M=N=K=8192, row-wise scales, no bias, bf16 out", "variant": "tiled"},
+        "roofline": {
+            "bound": "mfma",
+            "achieved": head["tflops"],
+            "peak": PEAK_FP8_TFLOPS,
+            "unit": "TFLOP/s",
+            "frac": head["tflops"] / PEAK_FP8_TFLOPS,
+            "traffic": None,
+        },
+    }
+
+    if not args.no_extra:
+        configs = {}
+        # C3: decode-sized, HBM-bound. Cold = rotate through operand sets larger than every cache.
+        cm, cn, ck = 16, 8192, 8192
+        cold_sets = make_device_inputs(cm, cn, ck, 1.0, False, dev, copies=10)
+        cold = figures(cm, cn, ck, False, time_steps_graph(cold_sets, 200, 5))
+        warm = figures(cm, cn, ck, False, time_steps_graph(cold_sets[:1], 200, 5))
+        configs["c3_skinny_16x8192x8192"] = {"cold": cold, "cache_resident": warm}
+        del cold_sets
+        line["hbm_metric"] = {
+            "metric": "fp8_gemm_rowwise HBM GB/s at M=16,N=K=8192 (cold operands)",
+            "value": cold["gbps"], "unit": "GB/s", "frac": cold["gbps"] / PEAK_HBM_GBPS,
+        }
+        for (rm, rn, rk) in [(1000, 3000, 4112), (4097, 7168, 2048)]:
+            rs = make_device_inputs(rm, rn, rk, 1.0, True, dev, copies=2)
+            configs[f"c5_ragged_bias_{rm}x{rn}x{rk}"] = figures(rm, rn, rk, True, time_steps_graph(rs, 50, 3))
+            del rs
+        configs["c2_square_8192_graph"] = figures(m, n, k, False, time_steps_graph(sets, 20, 2))
+        if args.all_configs:
+            for (ln, lk) in [(10240, 8192), (8192, 8192), (57344, 8192), (8192, 28672)]:
+                for lm in (1, 32, 128, 1024, 4096):
+                    copies = max(2, min(8, int(600e6 // (ln * lk)) + 1))
+                    ls = make_device_inputs(lm, ln, lk, 0.02, False, dev, copies=copies)
+                    configs[f"c4_llama70b_{lm}x{ln}x{lk}"] = figures(lm, ln, lk, False, time_steps_graph(ls, 30, 3))
+                    del ls
+                    torch.cuda.empty_cache()
+        line["configs"] = configs
+
+    if not args.no_cpu_baseline:
+        xq, wq, xs, ws, _, _ = sets[0]
+        line["cpu_baseline"] = cpu_baseline(xq, wq, xs, ws)
+
+    print(json.dumps(line))
+
+
+if __name__ == "__main__":
+    main()

@@ -90,10 +90,12 @@ int mi355x_fp8_rowwise_gemm(const void* a, const void* b,
 /*
  * Row-wise e4m3fn quantiser, replacing fp8_row_quantize (operator.py:136-145):
  *   amax[r]      = max_k |x[r,k]|
- *   scale[r]     = 448 / max(amax[r], 1e-12)
+ *   scale[r]     = fl(fl(1 / max(amax[r], 1e-12)) * 448)   (how PyTorch evaluates 448 / tensor)
  *   xq[r,k]      = e4m3fn( clamp(x[r,k] * scale[r], -448, 448) )     (round to nearest even)
  *   inv_scale[r] = 1 / scale[r]                                      (f32)
- * The arithmetic runs in f32 (a bf16 source is widened first).
+ * An f32 source is processed in f32. For a bf16 source every intermediate (scale, scaled
+ * value, inverse scale) is rounded to bf16, which is how eager PyTorch evaluates the same
+ * expression on a bf16 tensor. NaN inputs are not propagated (they quantise as +-448).
  *
  *   x  [R, K] of `src_type`, row stride ldx (elements)     xq  e4m3fn [R, K], row stride ldq
  */

@@ -1,0 +1,189 @@
+"""CPU restatement of the tritonbench `fp8_gemm_rowwise` path. TEST INFRASTRUCTURE ONLY
+(see oracle/__init__.py): the checker for tests/, smoke() and bench.py's cpu_baseline leg.
+
+What is restated, and from where (paths relative to the tritonbench checkout):
+  fp8_row_quantize      tritonbench/operators/fp8_gemm_rowwise/operator.py:130-145
+  dequant_matmul        the result the timed callables produce, operator.py:187-217, written as
+                        fp32 dequantise + matmul (the arithmetic itself lives in FBGEMM
+                        `fbgemm_gpu.experimental.gemm.triton_gemm.fp8_gemm.matmul_fp8_row` and
+                        `torch.ops.fbgemm.f8f8bf16_rowwise`; FBGEMM is an un-vendored, unpinned
+                        submodule of the checkout, so the published contract
+                        C = (A . B^T) * a_scale[:,None] * b_scale[None,:] + bias is restated)
+  flops / moved_bytes   operator.py:248-271
+  make_inputs           operator.py:280-297 (shapes, per-row A and per-row-of-[N,K] B
+                        quantisation, optional bf16 bias), seeded as utils/env_utils.py:20
+
+How each function is pinned (tests/test_oracle_*.py):
+  fp8_row_quantize      against an independent numpy restatement built on the bit-level
+                        codec of oracle/e4m3.py, against oracle/fp8_rowwise_ref.c, and through
+                        invariants (|xq| <= 448, max |xq| == 448 on non-zero rows, half-ulp
+                        reconstruction error, inverse scale is 1/(448/amax) bitwise)
+  dequant_matmul        against float64 brute force (gemm_f64, numpy) on small and ragged
+                        shapes, bit-exact integer cases, identity / one-hot operands, and
+                        oracle/fp8_rowwise_ref.c
+  matmul_fp8_row's own rounding / accumulation order and f8f8bf16_rowwise's CK instance
+  are NOT reproducible without FBGEMM: parity unpinned for those (the tolerance
+  rtol 1e-2 / atol 1e-2 is what absorbs them).
+"""
+import hashlib
+from typing import Optional, Tuple
+
+import numpy as np
+import torch
+
+from . import e4m3
+
+MAIN_RANDOM_SEED = 1337  # tritonbench/utils/env_utils.py:20
+FP8_DTYPE = torch.float8_e4m3fn
+E4M3_MAX_POS = torch.finfo(FP8_DTYPE).max  # 448.0, operator.py:131
+EPS = 1e-12  # operator.py:132
+FP16_MAX_POS = torch.finfo(torch.float16).max  # operator.py:133
+
+
+def fp8_row_quantize(x: torch.Tensor) -> Tuple[torch.Tensor, torch.Tensor]:
+    """operator.py:136-145. Arithmetic runs in x.dtype; returns (xq, 1/scale as f32).
+    Note `float / tensor` is evaluated by torch as `tensor.reciprocal() * float`, so
+    scale = fl(fl(1/amax) * 448), not the correctly rounded quotient."""
+    row_max = x.abs().max(dim=1).values
+    scale = E4M3_MAX_POS / row_max.clamp(min=EPS)
+    if x.dtype is torch.float16:
+        scale = scale.clamp(max=FP16_MAX_POS)
+    xq = (x * scale[:, None]).clamp(min=-E4M3_MAX_POS, max=E4M3_MAX_POS).to(FP8_DTYPE)
+    return xq, scale.reciprocal().to(torch.float32)
+
+
+def fp8_row_quantize_numpy(x: np.ndarray) -> Tuple[np.ndarray, np.ndarray]:
+    """Same computation for float32 input, in numpy with the bit-level codec; returns
+    (uint8 codes, f32 inverse scale). Exists to cross-check fp8_row_quantize."""
+    x = np.asarray(x, dtype=np.float32)
+    amax = np.max(np.abs(x), axis=1)
+    # torch evaluates `448.0 / tensor` as `tensor.reciprocal() * 448.0` (Tensor.__rtruediv__):
+    # two fp32 roundings, which is what the reference's `E4M3_MAX_POS / torch.clamp(...)` does
+    recip = (np.float32(1.0) / np.maximum(amax, np.float32(1e-12))).astype(np.float32)
+    scale = (recip * np.float32(448.0)).astype(np.float32)
+    y = (x * scale[:, None]).astype(np.float32)
+    y = np.minimum(np.maximum(y, np.float32(-448.0)), np.float32(448.0))
+    inv = (np.float32(1.0) / scale).astype(np.float32)
+    return e4m3.encode_rne(y), inv
+
+
+def dequant_matmul(
+    xq: torch.Tensor,
+    wq: torch.Tensor,
+    x_scale: torch.Tensor,
+    w_scale: torch.Tensor,
+    bias: Optional[torch.Tensor] = None,
+) -> torch.Tensor:
+    """The parity reference: fp32 dequantise-then-matmul on host cores, one bf16 rounding."""
+    a = xq.to(torch.float32) * x_scale[:, None]
+    b = wq.to(torch.float32) * w_scale[:, None]
+    out = a @ b.t()
+    if bias is not None:
+        out = out + bias.to(torch.float32)
+    return out.to(torch.bfloat16)
+
+
+def dequantize(q: torch.Tensor, scale: torch.Tensor) -> torch.Tensor:
+    """fp32 value of a row-wise quantised operand (one half of dequant_matmul)."""
+    return q.to(torch.float32) * scale[:, None]
+
+
+def dequant_matmul_rows(a_deq: torch.Tensor, b_deq: torch.Tensor, bias: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """dequant_matmul on operands already passed through dequantize(): lets a caller check
+    many row subsets against one dequantised weight without redoing the widening."""
+    out = a_deq @ b_deq.t()
+    if bias is not None:
+        out = out + bias.to(torch.float32)
+    return out.to(torch.bfloat16)
+
+
+def to_bf16_bits(x: np.ndarray) -> np.ndarray:
+    """float32 -> bf16 bit pattern (uint16), round to nearest even."""
+    u = np.asarray(x, dtype=np.float32).view(np.uint32).astype(np.uint64)
+    nan = np.isnan(x)
+    r = (u + 0x7FFF + ((u >> 16) & 1)) >> 16
+    r = np.where(nan, (u >> 16) | 0x40, r)
+    return r.astype(np.uint16)
+
+
+def bf16_bits_to_f32(b: np.ndarray) -> np.ndarray:
+    return (np.asarray(b, dtype=np.uint16).astype(np.uint32) << 16).view(np.float32)
+
+
+def gemm_f64(
+    a_codes: np.ndarray,
+    b_codes: np.ndarray,
+    a_scale: np.ndarray,
+    b_scale: np.ndarray,
+    bias_bf16_bits: Optional[np.ndarray] = None,
+) -> np.ndarray:
+    """Brute force in float64 from raw codes; returns float64 [M,N] BEFORE the bf16 rounding."""
+    a = e4m3.decode(a_codes).astype(np.float64)
+    b = e4m3.decode(b_codes).astype(np.float64)
+    out = (a @ b.T) * a_scale.astype(np.float64)[:, None] * b_scale.astype(np.float64)[None, :]
+    if bias_bf16_bits is not None:
+        out = out + bf16_bits_to_f32(bias_bf16_bits).astype(np.float64)[None, :]
+    return out
+
+
+def flops(m: int, n: int, k: int, bias: bool) -> int:
+    """operator.py:248-259."""
+    return 2 * m * n * k + (2 * m * n if bias else 0)
+
+
+def moved_bytes(m: int, n: int, k: int) -> int:
+    """operator.py:261-271: fp8 A + fp8 B + bf16 C (scales and bias not counted)."""
+    return m * k + n * k + 2 * m * n
+
+
+def _sub_seed(m: int, n: int, k: int, role: str) -> int:
+    h = hashlib.sha256(f"{MAIN_RANDOM_SEED}:{m}:{n}:{k}:{role}".encode()).digest()
+    return int.from_bytes(h[:7], "little")
+
+
+def randn_f32(rows: int, cols: int, sigma: float, seed: int) -> torch.Tensor:
+    g = torch.Generator(device="cpu")
+    g.manual_seed(seed)
+    x = torch.randn((rows, cols), generator=g, dtype=torch.float32)
+    if sigma != 1.0:
+        x.mul_(sigma)
+    return x
+
+
+def make_weight(n: int, k: int, sigma: float = 1.0):
+    """(wq, w_scale) for B [N,K]; depends only on (n, k) so an M sweep can reuse it."""
+    w = randn_f32(n, k, sigma, _sub_seed(0, n, k, "w"))
+    return fp8_row_quantize(w)
+
+
+def make_activation(m: int, n: int, k: int, sigma: float = 1.0):
+    x = randn_f32(m, k, sigma, _sub_seed(m, n, k, "x"))
+    return fp8_row_quantize(x)
+
+
+def make_bias(m: int, n: int, k: int, sigma: float = 0.1) -> torch.Tensor:
+    g = torch.Generator(device="cpu")
+    g.manual_seed(_sub_seed(m, n, k, "bias"))
+    return (sigma * torch.randn((n,), generator=g, dtype=torch.float32)).to(torch.bfloat16)
+
+
+def make_inputs(m: int, n: int, k: int, sigma: float = 1.0, bias: bool = False):
+    """Seeded host-side inputs (xq, wq, x_scale, w_scale, bias) as get_input_iter yields them."""
+    xq, x_scale = make_activation(m, n, k, sigma)
+    wq, w_scale = make_weight(n, k, sigma)
+    b = make_bias(m, n, k) if bias else None
+    return xq, wq, x_scale, w_scale, b
+
+
+# The five workload families the parity and bench code iterate over.
+LLAMA3_70B_NK = {"qkv": (10240, 8192), "o_proj": (8192, 8192), "gate_up": (57344, 8192), "down": (8192, 28672)}
+LLAMA3_70B_M = (1, 32, 128, 1024, 4096)
+CONFIGS = {
+    "c1_plumbing": dict(shapes=[(128, 256, 512)], sigma=1.0, bias=False),
+    "c2_square": dict(shapes=[(8192, 8192, 8192)], sigma=1.0, bias=False),
+    "c3_skinny": dict(shapes=[(16, 8192, 8192)], sigma=1.0, bias=False),
+    "c4_llama70b": dict(
+        shapes=[(m, n, k) for (n, k) in LLAMA3_70B_NK.values() for m in LLAMA3_70B_M], sigma=0.02, bias=False
+    ),
+    "c5_ragged_bias": dict(shapes=[(1000, 3000, 4112), (4097, 7168, 2048)], sigma=1.0, bias=True),
+}

@@ -1,0 +1,58 @@
+"""Writes the golden fixtures in this directory from the repository's own CPU oracle.
+
+The tritonbench checkout holds no golden vectors or known-answer tests for
+fp8_gemm_rowwise (the operator is skipped by its CI), so the vectors are produced here:
+seeded inputs, quantised by oracle.fp8_rowwise.fp8_row_quantize, outputs from
+oracle.fp8_rowwise.dequant_matmul. Each .npz holds raw arrays only (uint8 e4m3fn codes,
+float32 scales, uint16 bf16 bit patterns); load with allow_pickle=False.
+
+    python tests/golden/make_golden.py
+"""
+import hashlib
+import json
+import os
+import sys
+
+import numpy as np
+import torch
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, os.path.dirname(os.path.dirname(HERE)))
+
+from oracle import fp8_rowwise as orc  # noqa: E402
+
+CASES = [
+    # name, m, n, k, sigma, bias
+    ("c1_plumbing_128x256x512", 128, 256, 512, 1.0, False),
+    ("ragged_33x65x272_bias", 33, 65, 272, 1.0, True),
+    ("ragged_17x300x144", 17, 300, 144, 1.0, False),
+    ("decode_1x512x1024_sigma002", 1, 512, 1024, 0.02, False),
+    ("edge_257x259x400_bias", 257, 259, 400, 1.0, True),
+]
+
+
+def main():
+    manifest = {"generator": "tests/golden/make_golden.py", "seed": orc.MAIN_RANDOM_SEED, "cases": []}
+    for name, m, n, k, sigma, bias in CASES:
+        xq, wq, xs, ws, b = orc.make_inputs(m, n, k, sigma, bias)
+        out = orc.dequant_matmul(xq, wq, xs, ws, b)
+        arrays = dict(
+            a=xq.view(torch.uint8).numpy(),
+            b=wq.view(torch.uint8).numpy(),
+            a_scale=xs.numpy(),
+            b_scale=ws.numpy(),
+            c=out.view(torch.int16).numpy().view(np.uint16),
+        )
+        if bias:
+            arrays["bias"] = b.view(torch.int16).numpy().view(np.uint16)
+        fname = name + ".npz"
+        np.savez_compressed(os.path.join(HERE, fname), **arrays)
+        digest = hashlib.sha256(b"".join(np.ascontiguousarray(v).tobytes() for _, v in sorted(arrays.items()))).hexdigest()
+        manifest["cases"].append(dict(name=name, file=fname, m=m, n=n, k=k, sigma=sigma, bias=bias, sha256=digest))
+    with open(os.path.join(HERE, "manifest.json"), "w") as f:
+        json.dump(manifest, f, indent=1)
+    print(f"wrote {len(CASES)} cases")
+
+
+if __name__ == "__main__":
+    main()

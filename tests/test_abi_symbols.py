@@ -1,0 +1,62 @@
+"""The C-ABI library loads without a GPU and exports every function the header declares."""
+import ctypes
+import os
+import re
+
+from tritonbench_amd import _lib
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+HEADER = os.path.join(ROOT, "include", "mi355x_fp8_rowwise.h")
+
+
+def _declared_functions():
+    text = open(HEADER).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(mi355x_fp8_rowwise_\w+)\s*\(", text)))
+
+
+def test_header_declares_the_expected_entry_points():
+    assert _declared_functions() == sorted(_lib.SIGNATURES)
+
+
+def test_library_exports_every_declared_symbol():
+    lib = ctypes.CDLL(_lib.library_path())
+    for name in _declared_functions():
+        assert hasattr(lib, name), name
+
+
+def test_abi_version_and_status_constants_match_header():
+    text = open(HEADER).read()
+    consts = dict(re.findall(r"#define\s+(MI355X_FP8_\w+)\s+\(?(-?\d+)\)?", text))
+    assert int(consts["MI355X_FP8_ABI_VERSION"]) == _lib.ABI_VERSION == _lib.load().mi355x_fp8_rowwise_abi_version()
+    assert int(consts["MI355X_FP8_EINVAL"]) == _lib.EINVAL
+    assert int(consts["MI355X_FP8_ENOTSUP"]) == _lib.ENOTSUP
+    assert int(consts["MI355X_FP8_ELAUNCH"]) == _lib.ELAUNCH
+    assert int(consts["MI355X_FP8_VARIANT_TILED"]) == _lib.VARIANT_TILED
+    assert int(consts["MI355X_FP8_VARIANT_SKINNY"]) == _lib.VARIANT_SKINNY
+    assert int(consts["MI355X_FP8_SRC_BF16"]) == _lib.SRC_BF16
+
+
+def test_host_side_argument_checks_need_no_gpu():
+    lib = _lib.load()
+    # shape checks happen before anything touches a device
+    assert lib.mi355x_fp8_rowwise_select_variant(16, 8192, 8192) == _lib.VARIANT_SKINNY
+    assert lib.mi355x_fp8_rowwise_select_variant(8192, 8192, 8192) == _lib.VARIANT_TILED
+    assert lib.mi355x_fp8_rowwise_select_variant(0, 8, 16) == _lib.EINVAL
+    assert lib.mi355x_fp8_rowwise_select_variant(8, 8, 24) == _lib.ENOTSUP
+    assert "multiple of 16" in _lib.last_error()
+    st = lib.mi355x_fp8_rowwise_gemm(None, None, None, None, None, None, 16, 16, 16, 16, 16, 16, None, 0, 0, None)
+    assert st == _lib.EINVAL and "null" in _lib.last_error()
+    st = lib.mi355x_fp8_rowwise_gemm(None, None, None, None, None, None, 16, 16, 20, 32, 32, 16, None, 0, 0, None)
+    assert st == _lib.ENOTSUP
+
+
+def test_status_to_exception_mapping():
+    import pytest
+
+    lib = _lib.load()
+    with pytest.raises(NotImplementedError):
+        _lib.check(lib.mi355x_fp8_rowwise_select_variant(8, 8, 24), "select")
+    with pytest.raises(ValueError):
+        _lib.check(lib.mi355x_fp8_rowwise_select_variant(-1, 8, 16), "select")
+    _lib.check(0, "fine")

@@ -1,0 +1,109 @@
+"""The benchmark configurations at full size on the GPU, checked against the oracle evaluated
+on host cores for a sample of output rows (all columns), plus size-independent properties."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import fp8_rowwise as orc
+from tritonbench_amd import _lib, ops
+
+pytestmark = pytest.mark.gpu
+
+RTOL = 1e-2
+ATOL = 1e-2
+
+
+def _sample_rows(m, count=48):
+    edge = [0, 1, m - 1, m - 2, 255, 256, 257, 127, 128, m // 2]
+    rng = np.random.default_rng(m)
+    rows = sorted({r for r in edge if 0 <= r < m} | set(rng.integers(0, m, size=min(count, m)).tolist()))
+    return torch.tensor(rows, dtype=torch.long)
+
+
+def _check_rows(out, xq, wq, xs, ws, bias, rows, sigma, b_deq=None):
+    if b_deq is None:
+        want = orc.dequant_matmul(xq[rows], wq, xs[rows], ws, bias)
+    else:
+        want = orc.dequant_matmul_rows(orc.dequantize(xq[rows], xs[rows]), b_deq, bias)
+    got = out[rows.to(out.device)].cpu()
+    torch.testing.assert_close(got, want, rtol=RTOL, atol=ATOL)
+    # atol alone would pass almost anything when |C| is small (sigma = 0.02): also demand
+    # agreement to 2 bf16 ulp of the row's typical magnitude
+    g, w = got.float(), want.float()
+    scale = w.abs().mean(dim=1, keepdim=True).clamp_min(1e-30)
+    assert torch.all((g - w).abs() <= 2.0 ** -6 * scale + 2.0 ** -7 * w.abs()), "relative check failed"
+
+
+def _gpu(dev, *ts):
+    return [None if t is None else t.to(dev) for t in ts]
+
+
+def test_c2_square_8192(gpu_device):
+    m = n = k = 8192
+    xq, wq, xs, ws, _ = orc.make_inputs(m, n, k, 1.0, False)
+    dxq, dwq, dxs, dws = _gpu(gpu_device, xq, wq, xs, ws)
+    out = ops.fp8_gemm_rowwise(dxq, dwq, dxs, dws)
+    torch.cuda.synchronize()
+    _check_rows(out, xq, wq, xs, ws, None, _sample_rows(m), 1.0)
+    # linearity in the scales: doubling a_scale doubles every output exactly (power of two)
+    out2 = ops.fp8_gemm_rowwise(dxq, dwq, dxs * 2, dws)
+    torch.cuda.synchronize()
+    assert torch.equal(out2, out * 2)
+    # determinism: same launch, same bits
+    out3 = ops.fp8_gemm_rowwise(dxq, dwq, dxs, dws)
+    torch.cuda.synchronize()
+    assert torch.equal(out3, out)
+    # row permutation of A permutes rows of C
+    perm = torch.randperm(m, generator=torch.Generator().manual_seed(3)).to(gpu_device)
+    outp = ops.fp8_gemm_rowwise(dxq[perm].contiguous(), dwq, dxs[perm].contiguous(), dws)
+    torch.cuda.synchronize()
+    assert torch.equal(outp, out[perm])
+
+
+def test_c3_skinny_16x8192x8192(gpu_device):
+    m, n, k = 16, 8192, 8192
+    xq, wq, xs, ws, _ = orc.make_inputs(m, n, k, 1.0, False)
+    dxq, dwq, dxs, dws = _gpu(gpu_device, xq, wq, xs, ws)
+    out = ops.fp8_gemm_rowwise(dxq, dwq, dxs, dws)
+    torch.cuda.synchronize()
+    assert ops.select_variant(m, n, k) == _lib.VARIANT_SKINNY
+    _check_rows(out, xq, wq, xs, ws, None, torch.arange(m), 1.0)
+    # the two kernel families agree on the same inputs
+    out_t = ops.fp8_gemm_rowwise(dxq, dwq, dxs, dws, variant=_lib.VARIANT_TILED)
+    torch.cuda.synchronize()
+    torch.testing.assert_close(out_t, out, rtol=RTOL, atol=ATOL)
+
+
+@pytest.mark.parametrize("m,n,k", [(1000, 3000, 4112), (4097, 7168, 2048)])
+def test_c5_ragged_with_bias(gpu_device, m, n, k):
+    xq, wq, xs, ws, b = orc.make_inputs(m, n, k, 1.0, True)
+    dxq, dwq, dxs, dws, db = _gpu(gpu_device, xq, wq, xs, ws, b)
+    out = ops.fp8_gemm_rowwise(dxq, dwq, dxs, dws, bias=db)
+    torch.cuda.synchronize()
+    rows = torch.arange(m) if m <= 1000 else _sample_rows(m, 96)
+    _check_rows(out, xq, wq, xs, ws, b, rows, 1.0)
+    # bias is additive: result with bias minus result without, row by row, is the bias to
+    # within the two bf16 roundings
+    out0 = ops.fp8_gemm_rowwise(dxq, dwq, dxs, dws)
+    torch.cuda.synchronize()
+    diff = (out.float() - out0.float()).cpu()
+    tol = 2.0 ** -7 * (out.float().abs().cpu() + out0.float().abs().cpu()) + 1e-6
+    assert torch.all((diff - b.float()[None, :]).abs() <= tol)
+
+
+@pytest.mark.parametrize("name", list(orc.LLAMA3_70B_NK))
+def test_c4_llama70b_projections(gpu_device, name):
+    n, k = orc.LLAMA3_70B_NK[name]
+    sigma = 0.02
+    wq, ws = orc.make_weight(n, k, sigma)
+    dwq, dws = _gpu(gpu_device, wq, ws)
+    b_deq = orc.dequantize(wq, ws)
+    for m in orc.LLAMA3_70B_M:
+        print(f"llama {name} m={m} n={n} k={k}", flush=True)
+        xq, xs = orc.make_activation(m, n, k, sigma)
+        dxq, dxs = _gpu(gpu_device, xq, xs)
+        out = ops.fp8_gemm_rowwise(dxq, dwq, dxs, dws)
+        torch.cuda.synchronize()
+        rows = torch.arange(m) if m <= 32 else _sample_rows(m, 24 if n > 20000 else 48)
+        _check_rows(out, xq, wq, xs, ws, None, rows, sigma, b_deq)
+        del out, dxq, dxs

@@ -1,0 +1,309 @@
+"""Parity of the HIP path (through the C ABI) with the CPU oracle. Needs an MI355X."""
+import json
+import os
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import e4m3
+from oracle import fp8_rowwise as orc
+from tritonbench_amd import _lib, ops
+
+pytestmark = pytest.mark.gpu
+
+GOLDEN = os.path.join(os.path.dirname(__file__), "golden")
+RTOL = 1e-2  # the tolerance the path is specified to: rtol 1e-2 / atol 1e-2 on the bf16 output
+ATOL = 1e-2
+
+
+def _codes(t):
+    return t.view(torch.uint8).cpu().numpy()
+
+
+def _bits(t):
+    return t.view(torch.int16).cpu().numpy().view(np.uint16)
+
+
+def _ulp_bf16(x):
+    x = np.maximum(np.abs(x), 2.0 ** -126)
+    return 2.0 ** (np.floor(np.log2(x)) - 7)
+
+
+def _run(dev, xq, wq, xs, ws, bias=None, variant=_lib.VARIANT_AUTO):
+    d = lambda t: None if t is None else t.to(dev)
+    out = ops.fp8_gemm_rowwise(d(xq), d(wq), d(xs), d(ws), bias=d(bias), variant=variant)
+    torch.cuda.synchronize()
+    return out.cpu()
+
+
+def _check_tight(out, xq, wq, xs, ws, bias):
+    """Beyond rtol/atol: within 1 bf16 ulp of the exact (float64) value plus the slack any
+    fp32 accumulation order is entitled to. Keeps parity meaningful when |C| << atol."""
+    exact = orc.gemm_f64(_codes(xq), _codes(wq), xs.numpy(), ws.numpy(), _bits(bias) if bias is not None else None)
+    a = np.abs(e4m3.decode(_codes(xq)).astype(np.float64))
+    b = np.abs(e4m3.decode(_codes(wq)).astype(np.float64))
+    slack = (a @ b.T) * xs.numpy().astype(np.float64)[:, None] * ws.numpy().astype(np.float64)[None, :] * a.shape[1] * 2.0 ** -24
+    got = out.float().numpy().astype(np.float64)
+    err = np.abs(got - exact)
+    assert np.all(err <= 1.0 * _ulp_bf16(exact) + slack), f"max excess {np.max(err - _ulp_bf16(exact) - slack)}"
+
+
+VARIANTS = [_lib.VARIANT_AUTO, _lib.VARIANT_TILED, _lib.VARIANT_SKINNY]
+
+
+def test_golden_fixtures(gpu_device):
+    with open(os.path.join(GOLDEN, "manifest.json")) as f:
+        manifest = json.load(f)
+    for case in manifest["cases"]:
+        z = np.load(os.path.join(GOLDEN, case["file"]), allow_pickle=False)
+        xq = torch.from_numpy(z["a"]).view(torch.float8_e4m3fn)
+        wq = torch.from_numpy(z["b"]).view(torch.float8_e4m3fn)
+        xs, ws = torch.from_numpy(z["a_scale"]), torch.from_numpy(z["b_scale"])
+        bias = torch.from_numpy(z["bias"].view(np.int16)).view(torch.bfloat16) if case["bias"] else None
+        want = torch.from_numpy(z["c"].view(np.int16)).view(torch.bfloat16)
+        for variant in VARIANTS:
+            if variant == _lib.VARIANT_SKINNY and case["m"] > 64:
+                continue
+            print(f"golden {case['name']} variant {variant}", flush=True)
+            out = _run(gpu_device, xq, wq, xs, ws, bias, variant)
+            torch.testing.assert_close(out, want, rtol=RTOL, atol=ATOL)
+            _check_tight(out, xq, wq, xs, ws, bias)
+
+
+SMALL_SHAPES = [
+    # m, n, k, bias
+    (1, 1, 16, False), (1, 16, 16, True), (3, 5, 32, True), (16, 16, 128, False), (17, 33, 272, True),
+    (33, 17, 144, False), (64, 64, 64, True), (65, 63, 80, True), (100, 300, 1040, False),
+    (128, 256, 512, False), (255, 257, 384, True), (256, 256, 128, False), (257, 511, 4112, True),
+    (300, 200, 2048, False), (512, 768, 1024, True),
+]
+
+
+@pytest.mark.parametrize("m,n,k,bias", SMALL_SHAPES)
+@pytest.mark.parametrize("variant", VARIANTS)
+def test_seeded_shapes_against_oracle(gpu_device, m, n, k, bias, variant):
+    if variant == _lib.VARIANT_SKINNY and m > 64:
+        pytest.skip("skinny variant covers M <= 64")
+    print(f"case m={m} n={n} k={k} bias={bias} variant={variant}", flush=True)
+    xq, wq, xs, ws, b = orc.make_inputs(m, n, k, 1.0, bias)
+    want = orc.dequant_matmul(xq, wq, xs, ws, b)
+    out = _run(gpu_device, xq, wq, xs, ws, b, variant)
+    torch.testing.assert_close(out, want, rtol=RTOL, atol=ATOL)
+    _check_tight(out, xq, wq, xs, ws, b)
+
+
+@pytest.mark.parametrize("m", [1, 2, 15, 16, 17, 31, 32, 33, 47, 48, 49, 63, 64])
+def test_skinny_every_row_count(gpu_device, m):
+    n, k = 1000, 1168
+    xq, wq, xs, ws, b = orc.make_inputs(m, n, k, 0.02, True)
+    want = orc.dequant_matmul(xq, wq, xs, ws, b)
+    out = _run(gpu_device, xq, wq, xs, ws, b, _lib.VARIANT_SKINNY)
+    torch.testing.assert_close(out, want, rtol=RTOL, atol=ATOL)
+    _check_tight(out, xq, wq, xs, ws, b)
+
+
+@pytest.mark.parametrize("variant,m", [(_lib.VARIANT_TILED, 320), (_lib.VARIANT_SKINNY, 40)])
+def test_exact_integer_case_is_bit_exact(gpu_device, variant, m):
+    # small integers, unit scales: all partial sums < 2^24, fp32 accumulation is exact in any
+    # order, so the result must match the float64 computation bit for bit
+    rng = np.random.default_rng(11)
+    ints = np.array([0, 1, 2, 3, 4, -1, -2, -3, -4, 0.5, -0.5], dtype=np.float32)
+    n, k = 384, 1040
+    a = rng.choice(ints, size=(m, k)).astype(np.float32)
+    b = rng.choice(ints, size=(n, k)).astype(np.float32)
+    xq, wq = torch.from_numpy(a).to(torch.float8_e4m3fn), torch.from_numpy(b).to(torch.float8_e4m3fn)
+    out = _run(gpu_device, xq, wq, torch.ones(m), torch.ones(n), None, variant)
+    want = orc.to_bf16_bits((a.astype(np.float64) @ b.astype(np.float64).T).astype(np.float32))
+    assert np.array_equal(_bits(out), want)
+
+
+@pytest.mark.parametrize("variant,m", [(_lib.VARIANT_TILED, 300), (_lib.VARIANT_SKINNY, 20)])
+def test_every_code_pair_decodes_as_e4m3fn(gpu_device, variant, m):
+    # one-hot rows: C[i, j] = value(code_a[i]) * value(code_b[j]) exactly (products of two
+    # 4-bit significands fit fp32), so this pins the hardware's reading of every e4m3fn code,
+    # including 0x7e = 448, subnormals and negative zero
+    k = 16
+    finite = np.array([c for c in range(256) if (c & 0x7F) != 0x7F], dtype=np.uint8)
+    a_codes = np.zeros((m, k), dtype=np.uint8)
+    a_pick = finite[(np.arange(m) * 7) % len(finite)]
+    a_codes[:, 3] = a_pick
+    n = len(finite)
+    b_codes = np.zeros((n, k), dtype=np.uint8)
+    b_codes[:, 3] = finite
+    xq = torch.from_numpy(a_codes).view(torch.float8_e4m3fn)
+    wq = torch.from_numpy(b_codes).view(torch.float8_e4m3fn)
+    out = _run(gpu_device, xq, wq, torch.ones(m), torch.ones(n), None, variant)
+    t = e4m3.decode_table().astype(np.float64)
+    want = orc.to_bf16_bits((t[a_pick][:, None] * t[finite][None, :]).astype(np.float32))
+    got = _bits(out)
+    # +0 and -0 compare equal as values; compare bit patterns modulo the sign of zero
+    same = (got == want) | (((got | want) & 0x7FFF) == 0)
+    assert np.all(same)
+
+
+@pytest.mark.parametrize("variant,m", [(_lib.VARIANT_TILED, 270), (_lib.VARIANT_SKINNY, 33)])
+def test_one_hot_positions_catch_index_and_swizzle_errors(gpu_device, variant, m):
+    # A[i, ka(i)] = 1 and B[j, kb(j)] = 1: C[i, j] = [ka(i) == kb(j)]; walks every k residue
+    n, k = 290, 400
+    ka = (np.arange(m) * 37 + 5) % k
+    kb = (np.arange(n) * 11 + 2) % k
+    a = np.zeros((m, k), np.float32)
+    b = np.zeros((n, k), np.float32)
+    a[np.arange(m), ka] = 1.0
+    b[np.arange(n), kb] = 1.0
+    out = _run(gpu_device, torch.from_numpy(a).to(torch.float8_e4m3fn), torch.from_numpy(b).to(torch.float8_e4m3fn),
+               torch.ones(m), torch.ones(n), None, variant)
+    want = (ka[:, None] == kb[None, :]).astype(np.float32)
+    assert np.array_equal(out.float().numpy(), want)
+
+
+@pytest.mark.parametrize("variant,m", [(_lib.VARIANT_TILED, 130), (_lib.VARIANT_SKINNY, 9)])
+def test_identity_weight_and_scale_axes(gpu_device, variant, m):
+    k = 144
+    xq, _, xs, _, _ = orc.make_inputs(m, k, k, 1.0, False)
+    eye = torch.eye(k).to(torch.float8_e4m3fn)
+    ws = torch.linspace(0.5, 2.0, k)
+    out = _run(gpu_device, xq, eye, xs, ws, None, variant)
+    want = (xq.float() * xs[:, None] * ws[None, :]).to(torch.bfloat16)
+    # a single product chain in fp32: at most 1 ulp from the differently associated reference
+    assert np.all(np.abs(out.float().numpy() - want.float().numpy()) <= _ulp_bf16(want.float().numpy()))
+
+
+@pytest.mark.parametrize("variant,m", [(_lib.VARIANT_TILED, 200), (_lib.VARIANT_SKINNY, 24)])
+def test_padded_operands_and_output_canaries(gpu_device, variant, m):
+    # rows padded past K with garbage (lda, ldb > K), output embedded in a larger buffer:
+    # padding must not leak into sums and nothing outside C[M, N] may be written
+    n, k, pad = 150, 272, 48
+    xq, wq, xs, ws, b = orc.make_inputs(m, n, k, 1.0, True)
+    want = orc.dequant_matmul(xq, wq, xs, ws, b)
+    dev = gpu_device
+    a_buf = torch.full((m, k + pad), 0x7E, dtype=torch.uint8, device=dev)  # 448 everywhere
+    b_buf = torch.full((n, k + pad), 0xFE, dtype=torch.uint8, device=dev)  # -448 everywhere
+    a_buf[:, :k] = xq.view(torch.uint8).to(dev)
+    b_buf[:, :k] = wq.view(torch.uint8).to(dev)
+    c_buf = torch.full((m + 2, n + 24), -77.0, dtype=torch.bfloat16, device=dev)
+    c_view = c_buf[1:m + 1, 8:8 + n]
+    ops.fp8_gemm_rowwise(a_buf.view(torch.float8_e4m3fn)[:, :k], b_buf.view(torch.float8_e4m3fn)[:, :k],
+                         xs.to(dev), ws.to(dev), bias=b.to(dev), out=c_view, variant=variant)
+    torch.cuda.synchronize()
+    torch.testing.assert_close(c_view.cpu(), want, rtol=RTOL, atol=ATOL)
+    _check_tight(c_view.cpu(), xq, wq, xs, ws, b)
+    mask = torch.ones_like(c_buf, dtype=torch.bool)
+    mask[1:m + 1, 8:8 + n] = False
+    assert torch.all(c_buf[mask] == -77.0)
+
+
+def test_bias_is_fused_before_the_single_rounding(gpu_device):
+    a = torch.zeros(16, 16)
+    a[0, 0] = 1.0
+    b = torch.zeros(16, 16)
+    b[0, 0] = 1.0
+    xs = torch.ones(16)
+    xs[0] = 1.00390625
+    bias = torch.zeros(16)
+    bias[0] = 2.0 ** -8
+    for variant in (_lib.VARIANT_TILED, _lib.VARIANT_SKINNY):
+        out = _run(gpu_device, a.to(torch.float8_e4m3fn), b.to(torch.float8_e4m3fn), xs, torch.ones(16),
+                   bias.to(torch.bfloat16), variant)
+        assert out[0, 0].item() == 1.0078125
+
+
+def test_unsupported_and_invalid_arguments_raise(gpu_device):
+    dev = gpu_device
+    f8 = lambda *s: torch.zeros(*s, device=dev).to(torch.float8_e4m3fn)
+    with pytest.raises(NotImplementedError, match="multiple of 16"):
+        ops.fp8_gemm_rowwise(f8(16, 24), f8(16, 24), torch.ones(16, device=dev), torch.ones(16, device=dev))
+    with pytest.raises(NotImplementedError, match="skinny"):
+        ops.fp8_gemm_rowwise(f8(128, 32), f8(16, 32), torch.ones(128, device=dev), torch.ones(16, device=dev),
+                             variant=_lib.VARIANT_SKINNY)
+    with pytest.raises(TypeError):
+        ops.fp8_gemm_rowwise(torch.zeros(16, 16, device=dev), f8(16, 16), torch.ones(16, device=dev), torch.ones(16, device=dev))
+    with pytest.raises(ValueError):
+        ops.fp8_gemm_rowwise(f8(16, 16), f8(16, 32), torch.ones(16, device=dev), torch.ones(16, device=dev))
+    with pytest.raises(ValueError):
+        ops.fp8_gemm_rowwise(f8(16, 16), f8(16, 16), torch.ones(15, device=dev), torch.ones(16, device=dev))
+    with pytest.raises(ValueError, match="unknown variant"):
+        ops.fp8_gemm_rowwise(f8(16, 16), f8(16, 16), torch.ones(16, device=dev), torch.ones(16, device=dev), variant=99)
+
+
+def test_dispatch_is_pinned(gpu_device):
+    assert ops.select_variant(16, 8192, 8192) == _lib.VARIANT_SKINNY
+    assert ops.select_variant(64, 8192, 8192) == _lib.VARIANT_SKINNY
+    assert ops.select_variant(8192, 8192, 8192) == _lib.VARIANT_TILED
+
+
+def test_graph_capture_replays_match_eager(gpu_device):
+    # the benchmark harness times the callable inside a captured graph on a side stream
+    dev = gpu_device
+    for (m, n, k) in [(16, 2048, 2048), (300, 512, 1040)]:
+        xq, wq, xs, ws, b = orc.make_inputs(m, n, k, 1.0, True)
+        dxq, dwq, dxs, dws, db = (t.to(dev) for t in (xq, wq, xs, ws, b))
+        eager = ops.fp8_gemm_rowwise(dxq, dwq, dxs, dws, bias=db)
+        torch.cuda.synchronize()
+        out = torch.empty_like(eager)
+        stream = torch.cuda.Stream()
+        with torch.cuda.stream(stream):
+            ops.fp8_gemm_rowwise(dxq, dwq, dxs, dws, bias=db, out=out)  # warm-up outside capture
+            torch.cuda.synchronize()
+            g = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(g, stream=stream):
+                for _ in range(3):
+                    ops.fp8_gemm_rowwise(dxq, dwq, dxs, dws, bias=db, out=out)
+            for _ in range(3):
+                out.fill_(-5.0)
+                torch.cuda.synchronize()
+                g.replay()
+                torch.cuda.synchronize()
+                assert torch.equal(out, eager)
+
+
+# ---- quantiser ---------------------------------------------------------------------------
+@pytest.mark.parametrize("rows,cols,sigma", [(1, 16, 1.0), (7, 272, 1.0), (128, 512, 1.0), (33, 4112, 0.02), (1000, 1000, 3.0), (5, 17, 1.0)])
+def test_quantiser_fp32_bit_exact(gpu_device, rows, cols, sigma):
+    x = orc.randn_f32(rows, cols, sigma, seed=rows * 131 + cols)
+    want_q, want_inv = orc.fp8_row_quantize(x)
+    xq, inv = ops.fp8_row_quantize(x.to(gpu_device))
+    torch.cuda.synchronize()
+    assert torch.equal(xq.cpu().view(torch.uint8), want_q.view(torch.uint8))
+    assert torch.equal(inv.cpu().view(torch.int32), want_inv.view(torch.int32))
+
+
+@pytest.mark.parametrize("rows,cols", [(9, 144), (256, 2048)])
+def test_quantiser_bf16_bit_exact(gpu_device, rows, cols):
+    x = orc.randn_f32(rows, cols, 1.0, seed=rows + cols).to(torch.bfloat16)
+    want_q, want_inv = orc.fp8_row_quantize(x)
+    xq, inv = ops.fp8_row_quantize(x.to(gpu_device))
+    torch.cuda.synchronize()
+    assert torch.equal(xq.cpu().view(torch.uint8), want_q.view(torch.uint8))
+    assert torch.equal(inv.cpu().view(torch.int32), want_inv.view(torch.int32))
+
+
+def test_quantiser_special_rows(gpu_device):
+    x = torch.zeros(4, 64)
+    x[1, 5] = 1e-20
+    x[2, 7] = -3.0
+    x[3] = torch.linspace(-5e4, 5e4, 64)
+    want_q, want_inv = orc.fp8_row_quantize(x)
+    xq, inv = ops.fp8_row_quantize(x.to(gpu_device))
+    assert torch.equal(xq.cpu().view(torch.uint8), want_q.view(torch.uint8))
+    assert torch.equal(inv.cpu().view(torch.int32), want_inv.view(torch.int32))
+
+
+def test_quantise_then_gemm_end_to_end(gpu_device):
+    # fp32 -> HIP quantiser -> HIP GEMM, against the same chain in the oracle
+    m, n, k = 48, 640, 1024
+    x = orc.randn_f32(m, k, 1.0, seed=1)
+    w = orc.randn_f32(n, k, 1.0, seed=2)
+    oq, os_ = orc.fp8_row_quantize(x)
+    wq, ws = orc.fp8_row_quantize(w)
+    want = orc.dequant_matmul(oq, wq, os_, ws)
+    dxq, dxs = ops.fp8_row_quantize(x.to(gpu_device))
+    dwq, dws = ops.fp8_row_quantize(w.to(gpu_device))
+    out = ops.fp8_gemm_rowwise(dxq, dwq, dxs, dws)
+    torch.cuda.synchronize()
+    torch.testing.assert_close(out.cpu(), want, rtol=RTOL, atol=ATOL)
+    # and it approximates the unquantised product to fp8 accuracy
+    full = (x @ w.t())
+    rel = (out.cpu().float() - full).norm() / full.norm()
+    assert rel < 0.06

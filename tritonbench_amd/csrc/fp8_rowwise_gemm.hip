@@ -433,39 +433,45 @@ __device__ __forceinline__ uint8_t f32_to_e4m3fn_rne(float f) {
 }
 
 template <typename SrcT>
-__device__ __forceinline__ float load_src(const SrcT* p);
+struct SrcTraits;
+// fp32 source: every step rounds to fp32 once, as the eager PyTorch program does.
 template <>
-__device__ __forceinline__ float load_src<float>(const float* p) { return *p; }
+struct SrcTraits<float> {
+  static __device__ __forceinline__ float load(const float* p) { return *p; }
+  static __device__ __forceinline__ float round(float v) { return v; }
+};
+// bf16 source: PyTorch evaluates each elementwise op in fp32 and rounds its result back to
+// bf16, so amax, the scale, the scaled value and the inverse scale each pass through bf16.
 template <>
-__device__ __forceinline__ float load_src<uint16_t>(const uint16_t* p) { return bf16_to_f32(*p); }
+struct SrcTraits<uint16_t> {
+  static __device__ __forceinline__ float load(const uint16_t* p) { return bf16_to_f32(*p); }
+  static __device__ __forceinline__ float round(float v) { return bf16_to_f32(f32_to_bf16_rne(v)); }
+};
 
 template <typename SrcT>
 __global__ __launch_bounds__(256) void quantize_rows_kernel(const SrcT* x, uint8_t* xq,
                                                             float* inv_scale, int K, long ldx,
                                                             long ldq) {
+  using T = SrcTraits<SrcT>;
   __shared__ float wave_max[4];
   const long row = blockIdx.x;
   const SrcT* xr = x + row * ldx;
   uint8_t* qr = xq + row * ldq;
 
   float amax = 0.0f;
-  bool has_nan = false;
-  for (int k = threadIdx.x; k < K; k += 256) {
-    const float v = load_src<SrcT>(xr + k);
-    has_nan |= (v != v);
-    amax = fmaxf(amax, fabsf(v));
-  }
+  for (int k = threadIdx.x; k < K; k += 256) amax = fmaxf(amax, fabsf(T::load(xr + k)));
 #pragma unroll
   for (int o = 32; o > 0; o >>= 1) amax = fmaxf(amax, __shfl_xor(amax, o));
   if ((threadIdx.x & 63) == 0) wave_max[threadIdx.x >> 6] = amax;
   __syncthreads();
   amax = fmaxf(fmaxf(wave_max[0], wave_max[1]), fmaxf(wave_max[2], wave_max[3]));
-  (void)has_nan;
 
-  const float scale = 448.0f / fmaxf(amax, 1e-12f);
-  if (threadIdx.x == 0) inv_scale[row] = 1.0f / scale;
+  // `448.0 / tensor` in the PyTorch program this replaces evaluates as reciprocal * 448
+  const float recip = T::round(1.0f / fmaxf(amax, T::round(1e-12f)));
+  const float scale = T::round(recip * 448.0f);
+  if (threadIdx.x == 0) inv_scale[row] = T::round(1.0f / scale);
   for (int k = threadIdx.x; k < K; k += 256) {
-    float v = load_src<SrcT>(xr + k) * scale;
+    float v = T::round(T::load(xr + k) * scale);
     v = fminf(fmaxf(v, -448.0f), 448.0f);
     qr[k] = f32_to_e4m3fn_rne(v);
   }
