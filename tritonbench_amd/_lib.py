@@ -68,6 +68,12 @@ def load() -> ctypes.CDLL:
                 f"{LIB_PATH} does not exist; build it with `python -m tritonbench_amd.build` "
                 "(needs hipcc). There is no CPU or PyTorch fallback for this operator."
             )
+        # The library needs libamdhip64 by soname only. PyTorch-ROCm ships its own copy of the
+        # HIP runtime; whichever copy is mapped first serves the whole process, and two
+        # different copies cannot share a device. Importing torch first makes its runtime
+        # the one this library binds to, so torch streams and pointers are valid here.
+        import torch  # noqa: F401
+
         lib = ctypes.CDLL(LIB_PATH)
         for name, (restype, argtypes) in SIGNATURES.items():
             fn = getattr(lib, name)  # AttributeError if the symbol is missing
