@@ -21,6 +21,7 @@
 #include <stdarg.h>
 #include <stdio.h>
 #include <string.h>
+#include <type_traits>
 
 #include "../../include/mi355x_fp8_rowwise.h"
 
@@ -31,10 +32,11 @@ typedef int   v8i  __attribute__((ext_vector_type(8)));
 typedef float v4f  __attribute__((ext_vector_type(4)));
 typedef float v16f __attribute__((ext_vector_type(16)));
 typedef unsigned short us4 __attribute__((ext_vector_type(4)));
+typedef unsigned int v2u __attribute__((ext_vector_type(2)));
 
 constexpr int kNumXcd = 8;       // accelerator complex dies; workgroup ids round-robin over them
 constexpr int kNumCu = 256;
-constexpr int kBK = 128;         // bytes (= fp8 elements) of K per LDS stage
+constexpr int kBK = 128;         // bytes (= fp8 elements) of K one 16x16x128 MFMA consumes (skinny kernel step)
 constexpr int kChunk = 16;       // bytes moved per lane per load
 
 struct GemmParams {
@@ -59,6 +61,14 @@ __device__ __forceinline__ uint16_t f32_to_bf16_rne(float f) {
 
 __device__ __forceinline__ float bf16_to_f32(uint16_t h) {
   return __uint_as_float(((uint32_t)h) << 16);
+}
+
+// Two f32 -> two bf16 (round to nearest even, NaN kept) in one gfx950 instruction;
+// `lo` lands in bits 0..15.
+__device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi) {
+  uint32_t r;
+  asm("v_cvt_pk_bf16_f32 %0, %1, %2" : "=v"(r) : "v"(lo), "v"(hi));
+  return r;
 }
 
 // ------------------------------------------------------------------------------------
@@ -97,15 +107,19 @@ __device__ __forceinline__ void tile_coords(int t, int tiles_m, int tiles_n, int
 }
 
 // ------------------------------------------------------------------------------------
-// LDS tile layout. A stage holds BM rows of A then BN rows of B, 128 bytes per row, i.e. 8
-// chunks of 16 bytes. Chunk c of row r is kept at chunk position c ^ swz(r) so that the
-// MFMA operand reads (consecutive lanes = consecutive rows, same logical chunk) spread
-// over all banks instead of piling onto one.
+// LDS layout of the tiled kernel. A "stage" of an operand holds a 128-byte K slab of the
+// tile's rows: 128 bytes per row = 8 chunks of 16 bytes, fetched from global memory as whole
+// 128-byte lines. Chunk c of row r sits at chunk position c ^ ((r >> 1) & 7): the MFMA
+// operand reads (consecutive lanes = consecutive rows, same logical chunk) then spread over
+// all banks. A has two stages, B three (2*32 KB + 3*32 KB = all 160 KB of a 256x256 tile's
+// LDS): the A loads of a step are the only ones that must arrive within one step, and they
+// are issued first, so at most half of every load burst is urgent.
 // ------------------------------------------------------------------------------------
-template <int SWZ_SHIFT>
-__device__ __forceinline__ int swz(int row) {
-  return (row >> SWZ_SHIFT) & 7;
-}
+constexpr int kStepK = 128;
+constexpr int kStagesA = 2;
+constexpr int kStagesB = 3;
+
+__device__ __forceinline__ int swz128(int row) { return (row >> 1) & 7; }
 
 __device__ __forceinline__ void load_chunk_to_lds(const uint8_t* gsrc, uint8_t* lds_wave_base) {
   // Each lane fetches 16 bytes; the hardware deposits lane i's bytes at lds_wave_base + 16*i.
@@ -114,17 +128,52 @@ __device__ __forceinline__ void load_chunk_to_lds(const uint8_t* gsrc, uint8_t* 
       (__attribute__((address_space(3))) void*)lds_wave_base, 16, 0, 0);
 }
 
-template <int BM, int BN, int WAVES_M, int WAVES_N, int SWZ_SHIFT>
+// Scheduling hints for the machine scheduler: MFMA / LDS read / global load slots.
+#define SCHED_MFMA(n) __builtin_amdgcn_sched_group_barrier(0x008, n, 0)
+#define SCHED_DSREAD(n) __builtin_amdgcn_sched_group_barrier(0x100, n, 0)
+#define SCHED_VMEM(n) __builtin_amdgcn_sched_group_barrier(0x020, n, 0)
+
+// Waits until at most VM of this wave's global loads and none of its LDS operations are
+// outstanding, then joins the workgroup barrier. Written with the s_waitcnt builtin (not
+// inline asm) so the compiler's own wait-count bookkeeping knows the LDS queue is empty
+// afterwards and does not add full waits in front of the MFMAs that follow.
+template <int VM>
+__device__ __forceinline__ void wait_loads_and_barrier() {
+  // gfx9 encoding: vmcnt[3:0] | expcnt[6:4] | lgkmcnt[11:8] | vmcnt[5:4] at [15:14]
+  constexpr int imm = (VM & 15) | ((VM >> 4) << 14) | (7 << 4) | (0 << 8);
+  __builtin_amdgcn_s_waitcnt(imm);
+  __builtin_amdgcn_s_barrier();
+}
+
+// Cursor over the (tile, K step) sequence a workgroup walks; one for the A loads, one for
+// the B loads (which run a step further ahead).
+struct StepCursor {
+  int tile, kt, issued;
+};
+
+// The kernel is one software pipeline over "steps" (a 128-byte K slab of one tile) that runs
+// through all tiles a workgroup owns without draining at tile boundaries. For step g:
+//
+//   [A] LDS reads of (g, second K half) interleaved with the MFMAs of (g, first K half)
+//       wait for own loads of A(g+1) and B(g+1); workgroup barrier
+//   [B] issue loads A(g+2) and B(g+3) into the stages step g just released;
+//       LDS reads of (g+1, first half) interleaved with the MFMAs of (g, second half)
+//   after a tile's last step: epilogue (loads of the next tile are already in flight)
+//
+// Two register sets of operand fragments alternate between the halves; one barrier per step.
+template <int BM, int BN, int WAVES_M, int WAVES_N, bool KTAIL, bool HAS_BIAS>
 __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_tiled_kernel(GemmParams p) {
   constexpr int NW = WAVES_M * WAVES_N;
   constexpr int WTM = BM / WAVES_M;    // wave tile rows (m)
   constexpr int WTN = BN / WAVES_N;    // wave tile cols (n)
   constexpr int MT = WTM / 32, NT = WTN / 32;
-  constexpr int STAGE = (BM + BN) * kBK;
-  constexpr int A_GROUPS = BM / 8 / NW;  // 8-row groups of A each wave fetches per stage
+  constexpr int STAGE_A = BM * kStepK, STAGE_B = BN * kStepK;
+  constexpr int LDS_B0 = kStagesA * STAGE_A;  // B stages follow the A stages
+  constexpr int A_GROUPS = BM / 8 / NW;       // 8-row groups (1 KB of LDS) each wave fetches per step
   constexpr int B_GROUPS = BN / 8 / NW;
   static_assert(BM % (8 * NW) == 0 && BN % (8 * NW) == 0, "tile rows must split over waves");
   static_assert(WTM % 32 == 0 && WTN % 32 == 0, "wave tile must be a multiple of 32x32");
+  static_assert(A_GROUPS + 2 * B_GROUPS < 64, "outstanding-load count must fit the vmcnt field");
 
   extern __shared__ __attribute__((aligned(1024))) uint8_t lds[];
 
@@ -133,167 +182,305 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_tiled_kernel(GemmP
   const int wm = wave / WAVES_N, wn = wave % WAVES_N;
   const int l32 = lane & 31, half = lane >> 5;
 
-  // ---- per-lane constants of the global->LDS copy
-  const int ld_row = lane >> 3;  // row inside an 8-row group
-  const int ld_pc = lane & 7;    // physical chunk this lane's 16 bytes land in
+  // ---- per-lane constants of the global->LDS copy: a wave-wide load fills 8 rows
+  const int ld_row = lane >> 3;
+  const int ld_pc = lane & 7;  // physical chunk this lane's 16 bytes land in
+  // 8*group + ld_row: the swizzle key depends on ld_row and the parity of the group only
+  auto ld_chunk_off = [&](int group) { return (ld_pc ^ swz128(group * 8 + ld_row)) * kChunk; };
 
-  // ---- per-lane constants of the LDS->register operand reads
-  // Lane (l32, half) takes, for K sub-step s (64 bytes) and j in {0,1}, logical chunk
-  // 4*half + 2*s + j of its row. Any assignment is valid as long as A and B use the same
-  // one; this one keeps the two halves of the wave in different 64-byte halves of a row.
+  // ---- per-lane constants of the LDS->register operand reads. For K half s (64 bytes) and
+  // j in {0,1}, lane (l32, half) takes logical chunk 4*half + 2*s + j of its row. Any
+  // assignment is valid as long as A and B use the same one; this one keeps the two halves
+  // of the wave in different 64-byte halves of a row.
   int rd_off[2][2];
 #pragma unroll
   for (int s = 0; s < 2; ++s)
 #pragma unroll
     for (int j = 0; j < 2; ++j)
-      rd_off[s][j] = l32 * kBK + (((4 * half + 2 * s + j) ^ swz<SWZ_SHIFT>(l32)) * kChunk);
-  const int a_rd_base = (wm * WTM) * kBK;
-  const int b_rd_base = BM * kBK + (wn * WTN) * kBK;
+      rd_off[s][j] = l32 * kStepK + (((4 * half + 2 * s + j) ^ swz128(l32)) * kChunk);
+  const int a_rd_base = (wm * WTM) * kStepK;
+  const int b_rd_base = LDS_B0 + (wn * WTN) * kStepK;
 
   const int total_tiles = p.tiles_m * p.tiles_n;
   const TileWalk walk = make_walk(total_tiles);
-  const int k_full = p.K / kBK;            // whole 128-byte steps
-  const int k_tail = p.K - k_full * kBK;   // 0 or a multiple of 16
+  if (walk.slot >= walk.chunk_len) return;  // uniform over the workgroup
+  const int my_tiles = (walk.chunk_len - walk.slot + walk.slots - 1) / walk.slots;
+  const int k_full = p.K / kStepK;             // whole 128-byte steps
+  const int k_tail = p.K - k_full * kStepK;    // 0 or a multiple of 16
   const int k_steps = k_full + (k_tail ? 1 : 0);
+  const int total_steps = my_tiles * k_steps;
 
-  for (int li = walk.slot; li < walk.chunk_len; li += walk.slots) {
+  // ---- load side of the pipeline
+  StepCursor ca = {walk.slot, 0, 0}, cb = {walk.slot, 0, 0};
+  const uint8_t* l_a = nullptr;
+  const uint8_t* l_b = nullptr;
+  uint32_t a_off[A_GROUPS], b_off[B_GROUPS];
+  // Rows past the matrix edge are redirected to the last valid row: they are read but never
+  // stored, so every load stays in bounds without predication.
+  auto setup_a = [&](int li) {
     int tm, tn;
     tile_coords(walk.chunk_begin + li, p.tiles_m, p.tiles_n, p.group_m, tm, tn);
-    const int m0 = tm * BM, n0 = tn * BN;
-
-    // Rows past the matrix edge are redirected to the last valid row: they are read but
-    // never stored, so every load stays in bounds without predication.
-    uint32_t a_off[A_GROUPS], b_off[B_GROUPS];
-    const uint8_t* a_tile = p.a + (size_t)m0 * p.lda;
-    const uint8_t* b_tile = p.b + (size_t)n0 * p.ldb;
+    const int m0 = tm * BM;
+    l_a = p.a + (size_t)m0 * p.lda;
 #pragma unroll
     for (int i = 0; i < A_GROUPS; ++i) {
-      const int r = (wave + NW * i) * 8 + ld_row;
-      const int rc = min(r, p.M - 1 - m0);
-      a_off[i] = (uint32_t)rc * (uint32_t)p.lda + ((ld_pc ^ swz<SWZ_SHIFT>(r)) * kChunk);
+      const int grp = wave + NW * i;
+      a_off[i] = (uint32_t)min(grp * 8 + ld_row, p.M - 1 - m0) * (uint32_t)p.lda + ld_chunk_off(grp);
     }
+  };
+  auto setup_b = [&](int li) {
+    int tm, tn;
+    tile_coords(walk.chunk_begin + li, p.tiles_m, p.tiles_n, p.group_m, tm, tn);
+    const int n0 = tn * BN;
+    l_b = p.b + (size_t)n0 * p.ldb;
 #pragma unroll
     for (int i = 0; i < B_GROUPS; ++i) {
-      const int r = (wave + NW * i) * 8 + ld_row;
-      const int rc = min(r, p.N - 1 - n0);
-      b_off[i] = (uint32_t)rc * (uint32_t)p.ldb + ((ld_pc ^ swz<SWZ_SHIFT>(r)) * kChunk);
+      const int grp = wave + NW * i;
+      b_off[i] = (uint32_t)min(grp * 8 + ld_row, p.N - 1 - n0) * (uint32_t)p.ldb + ld_chunk_off(grp);
     }
-
-    auto issue_stage = [&](int kt, int stage) {
-      uint8_t* sbase = lds + stage * STAGE;
-      const size_t kb = (size_t)kt * kBK;
-      if (kt < k_full) {
+  };
+  // Issues one operand's loads for its cursor's step into stage (issued % STAGES). Past the
+  // last step it re-issues the last one into a stage nobody reads again, which keeps the
+  // path free of branches.
+  auto issue = [&](const uint8_t* gbase, const uint32_t* off, int groups, int kt, uint8_t* sbase) {
+    const uint8_t* g = gbase + (size_t)kt * kStepK;
+    if (!KTAIL || kt < k_full) {
 #pragma unroll
-        for (int i = 0; i < A_GROUPS; ++i)
-          load_chunk_to_lds(a_tile + kb + a_off[i], sbase + (wave + NW * i) * 1024);
+      for (int i = 0; i < A_GROUPS; ++i)
+        if (i < groups) load_chunk_to_lds(g + off[i], sbase + (wave + NW * i) * 1024);
+    } else {
+      // K tail: chunks at or past K are written as zeros (they would pollute the sums)
 #pragma unroll
-        for (int i = 0; i < B_GROUPS; ++i)
-          load_chunk_to_lds(b_tile + kb + b_off[i], sbase + BM * kBK + (wave + NW * i) * 1024);
-      } else {
-        // K tail: chunks past K are written as zeros (they would otherwise pollute the sums).
-#pragma unroll
-        for (int i = 0; i < A_GROUPS; ++i) {
-          const int r = (wave + NW * i) * 8 + ld_row;
-          const int c = ld_pc ^ swz<SWZ_SHIFT>(r);
-          v4i v = {0, 0, 0, 0};
-          if (c * kChunk < k_tail) v = *(const v4i*)(a_tile + kb + a_off[i]);
-          *(v4i*)(sbase + (wave + NW * i) * 1024 + lane * kChunk) = v;
-        }
-#pragma unroll
-        for (int i = 0; i < B_GROUPS; ++i) {
-          const int r = (wave + NW * i) * 8 + ld_row;
-          const int c = ld_pc ^ swz<SWZ_SHIFT>(r);
-          v4i v = {0, 0, 0, 0};
-          if (c * kChunk < k_tail) v = *(const v4i*)(b_tile + kb + b_off[i]);
-          *(v4i*)(sbase + BM * kBK + (wave + NW * i) * 1024 + lane * kChunk) = v;
-        }
-      }
-    };
-
-    v16f acc[MT][NT];
-#pragma unroll
-    for (int i = 0; i < MT; ++i)
-#pragma unroll
-      for (int j = 0; j < NT; ++j)
-#pragma unroll
-        for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.0f;
-
-    __syncthreads();  // previous tile's readers are done with both stages
-    issue_stage(0, 0);
-
-    for (int kt = 0; kt < k_steps; ++kt) {
-      const int stage = kt & 1;
-      __syncthreads();  // stage `stage` has landed everywhere; the other stage is free
-      if (kt + 1 < k_steps) issue_stage(kt + 1, stage ^ 1);
-
-      const uint8_t* sa = lds + stage * STAGE + a_rd_base;
-      const uint8_t* sb = lds + stage * STAGE + b_rd_base;
-#pragma unroll
-      for (int s = 0; s < 2; ++s) {
-        v8i af[MT], bf[NT];
-#pragma unroll
-        for (int i = 0; i < MT; ++i) {
-          const v4i lo = *(const v4i*)(sa + i * 32 * kBK + rd_off[s][0]);
-          const v4i hi = *(const v4i*)(sa + i * 32 * kBK + rd_off[s][1]);
-          af[i] = (v8i){lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
-        }
-#pragma unroll
-        for (int j = 0; j < NT; ++j) {
-          const v4i lo = *(const v4i*)(sb + j * 32 * kBK + rd_off[s][0]);
-          const v4i hi = *(const v4i*)(sb + j * 32 * kBK + rd_off[s][1]);
-          bf[j] = (v8i){lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
-        }
-#pragma unroll
-        for (int i = 0; i < MT; ++i)
-#pragma unroll
-          for (int j = 0; j < NT; ++j)
-            acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(
-                bf[j], af[i], acc[i][j], 0, 0, 0, 0, 0, 0);
+      for (int i = 0; i < A_GROUPS; ++i) {
+        if (i >= groups) continue;
+        const int c = ld_pc ^ swz128((wave + NW * i) * 8 + ld_row);
+        v4i v = {0, 0, 0, 0};
+        if (c * kChunk < k_tail) v = *(const v4i*)(g + off[i]);
+        *(v4i*)(sbase + (wave + NW * i) * 1024 + lane * kChunk) = v;
       }
     }
+  };
+  static_assert(A_GROUPS == B_GROUPS, "issue() unrolls over A_GROUPS for both operands");
+  auto issue_a = [&]() {
+    issue(l_a, a_off, A_GROUPS, ca.kt, lds + (ca.issued % kStagesA) * STAGE_A);
+    ++ca.issued;
+  };
+  auto issue_b = [&]() {
+    issue(l_b, b_off, B_GROUPS, cb.kt, lds + LDS_B0 + (cb.issued % kStagesB) * STAGE_B);
+    ++cb.issued;
+  };
+  auto advance_a = [&]() {
+    if (ca.issued >= total_steps) return;  // stay on the last step
+    if (++ca.kt == k_steps) {
+      ca.kt = 0;
+      ca.tile += walk.slots;
+      setup_a(ca.tile);
+    }
+  };
+  auto advance_b = [&]() {
+    if (cb.issued >= total_steps) return;
+    if (++cb.kt == k_steps) {
+      cb.kt = 0;
+      cb.tile += walk.slots;
+      setup_b(cb.tile);
+    }
+  };
 
-    // ---- epilogue: lane holds, for every (i, j) sub-tile, row m = .. + l32 and the columns
-    // n = .. + 8*q + 4*half + e (register v = 4*q + e).
-    const bool full = (m0 + BM <= p.M) && (n0 + BN <= p.N) && ((p.ldc & 3) == 0) &&
-                      ((reinterpret_cast<uintptr_t>(p.c) & 7) == 0);
+  // ---- operand fragments: two register sets; each fragment is two 16-byte LDS reads
+  struct Frag {
+    v4i lo, hi;
+  };
+  Frag xa[MT], xb[NT], ya[MT], yb[NT];
+  auto read_lo = [&](const uint8_t* rows, int s, int i) -> v4i {
+    return *(const v4i*)(rows + i * 32 * kStepK + rd_off[s][0]);
+  };
+  auto read_hi = [&](const uint8_t* rows, int s, int i) -> v4i {
+    return *(const v4i*)(rows + i * 32 * kStepK + rd_off[s][1]);
+  };
+  auto as_v8 = [](const Frag& f) -> v8i {
+    return (v8i){f.lo[0], f.lo[1], f.lo[2], f.lo[3], f.hi[0], f.hi[1], f.hi[2], f.hi[3]};
+  };
+
+  v16f acc[MT][NT];
 #pragma unroll
-    for (int i = 0; i < MT; ++i) {
-      const int m = m0 + wm * WTM + i * 32 + l32;
-      const float sa_m = p.a_scale[min(m, p.M - 1)];
-      uint16_t* crow = p.c + (size_t)m * p.ldc;
+  for (int i = 0; i < MT; ++i)
 #pragma unroll
-      for (int j = 0; j < NT; ++j) {
+    for (int j = 0; j < NT; ++j)
 #pragma unroll
-        for (int q = 0; q < 4; ++q) {
-          const int n = n0 + wn * WTN + j * 32 + 8 * q + 4 * half;
-          if (full) {
-            const v4f sb4 = *(const v4f*)(p.b_scale + n);
-            float r[4];
+      for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.0f;
+
+  // t-th MFMA of a half step (t = i*NT + j) on fragment set (fa, fb)
+  auto mfma_one = [&](const Frag (&fa)[MT], const Frag (&fb)[NT], int t) {
+    const int i = t / NT, j = t % NT;
+    acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(as_v8(fb[j]), as_v8(fa[i]), acc[i][j], 0, 0, 0, 0, 0, 0);
+  };
+  // u-th of the 2*(MT+NT) LDS reads that fill fragment set (fa, fb) with K half s
+  auto read_one = [&](Frag (&fa)[MT], Frag (&fb)[NT], const uint8_t* rows_a, const uint8_t* rows_b, int s, int u) {
+    const int f = u >> 1;
+    if (f < MT) {
+      if (u & 1) fa[f].hi = read_hi(rows_a, s, f);
+      else fa[f].lo = read_lo(rows_a, s, f);
+    } else {
+      if (u & 1) fb[f - MT].hi = read_hi(rows_b, s, f - MT);
+      else fb[f - MT].lo = read_lo(rows_b, s, f - MT);
+    }
+  };
+  constexpr int NMFMA = MT * NT, NREAD = 2 * (MT + NT), NLOAD = A_GROUPS + B_GROUPS;
+  static_assert(NREAD <= NMFMA && NLOAD <= NMFMA, "one read and one load slot per MFMA");
+
+  // ---- prologue: A(0) B(0) A(1) B(1) B(2) in flight, first fragments in registers
+  setup_a(ca.tile);
+  setup_b(cb.tile);
+  issue_a(); advance_a();
+  issue_b(); advance_b();
+  issue_a(); advance_a();
+  issue_b(); advance_b();
+  issue_b(); advance_b();
+  if (KTAIL) wait_loads_and_barrier<0>();
+  else wait_loads_and_barrier<A_GROUPS + 2 * B_GROUPS>();
 #pragma unroll
-            for (int e = 0; e < 4; ++e) r[e] = acc[i][j][4 * q + e] * sa_m * sb4[e];
-            if (p.bias) {
-              const us4 b4 = *(const us4*)(p.bias + n);
+  for (int u = 0; u < NREAD; ++u) read_one(xa, xb, lds + a_rd_base, lds + b_rd_base, 0, u);
+
+  // ---- epilogue. For every (i, j) sub-tile the lane holds row m = .. + l32 and the columns
+  // n = .. + 8*q + 4*half + e (register v = 4*q + e). All scale and bias values the lane
+  // needs are fetched up front (one memory latency per tile), then each sub-tile is scaled,
+  // rounded to bf16 by the hardware pack-convert and stored; INTERIOR tiles use 8-byte
+  // stores, edge tiles guard every element. Accumulators are cleared on the way out.
+  auto epilogue = [&](int m0, int n0, auto interior_tag) {
+    constexpr bool INTERIOR = decltype(interior_tag)::value;
+    float sam[MT], sbn[NT][4][4], bn[NT][4][4];
 #pragma unroll
-              for (int e = 0; e < 4; ++e) r[e] += bf16_to_f32(b4[e]);
-            }
-            us4 o;
+    for (int i = 0; i < MT; ++i) sam[i] = p.a_scale[min(m0 + wm * WTM + i * 32 + l32, p.M - 1)];
 #pragma unroll
-            for (int e = 0; e < 4; ++e) o[e] = f32_to_bf16_rne(r[e]);
-            *(us4*)(crow + n) = o;
-          } else if (m < p.M) {
+    for (int j = 0; j < NT; ++j)
 #pragma unroll
-            for (int e = 0; e < 4; ++e) {
-              if (n + e < p.N) {
-                float r = acc[i][j][4 * q + e] * sa_m * p.b_scale[n + e];
-                if (p.bias) r += bf16_to_f32(p.bias[n + e]);
-                crow[n + e] = f32_to_bf16_rne(r);
-              }
-            }
+      for (int q = 0; q < 4; ++q) {
+        const int n = n0 + wn * WTN + j * 32 + 8 * q + 4 * half;
+        if (INTERIOR) {
+          const v4f s4 = *(const v4f*)(p.b_scale + n);
+#pragma unroll
+          for (int e = 0; e < 4; ++e) sbn[j][q][e] = s4[e];
+          if (HAS_BIAS) {
+            const us4 b4 = *(const us4*)(p.bias + n);
+#pragma unroll
+            for (int e = 0; e < 4; ++e) bn[j][q][e] = bf16_to_f32(b4[e]);
+          }
+        } else {
+#pragma unroll
+          for (int e = 0; e < 4; ++e) {
+            sbn[j][q][e] = p.b_scale[min(n + e, p.N - 1)];
+            if (HAS_BIAS) bn[j][q][e] = bf16_to_f32(p.bias[min(n + e, p.N - 1)]);
           }
         }
       }
+#pragma unroll
+    for (int i = 0; i < MT; ++i) {
+      const int m = m0 + wm * WTM + i * 32 + l32;
+      uint16_t* crow = p.c + (size_t)m * p.ldc + n0 + wn * WTN + 4 * half;
+#pragma unroll
+      for (int j = 0; j < NT; ++j) {
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          float r[4];
+#pragma unroll
+          for (int e = 0; e < 4; ++e) {
+            const float t = acc[i][j][4 * q + e] * sam[i];
+            r[e] = HAS_BIAS ? __builtin_fmaf(t, sbn[j][q][e], bn[j][q][e]) : t * sbn[j][q][e];
+          }
+          const uint32_t lo = pack_bf16x2(r[0], r[1]), hi = pack_bf16x2(r[2], r[3]);
+          uint16_t* dst = crow + j * 32 + 8 * q;
+          if (INTERIOR) {
+            *(v2u*)dst = (v2u){lo, hi};
+          } else if (m < p.M) {
+            const int n = n0 + wn * WTN + j * 32 + 8 * q + 4 * half;
+            if (n + 0 < p.N) dst[0] = (uint16_t)lo;
+            if (n + 1 < p.N) dst[1] = (uint16_t)(lo >> 16);
+            if (n + 2 < p.N) dst[2] = (uint16_t)hi;
+            if (n + 3 < p.N) dst[3] = (uint16_t)(hi >> 16);
+          }
+        }
+#pragma unroll
+        for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.0f;
+      }
+    }
+    __builtin_amdgcn_sched_barrier(0);
+  };
+
+  int sa = 0, sb = 0;  // stages holding the step being computed
+  // Tile loop around the K loop (rather than one flat loop with a conditional epilogue):
+  // the accumulators then have one simple live range per tile, which the register
+  // allocator keeps in place.
+  for (int c_tile = walk.slot; c_tile < walk.chunk_len; c_tile += walk.slots) {
+    for (int kt = 0; kt < k_steps; ++kt) {
+      const uint8_t* cur_a = lds + a_rd_base + sa * STAGE_A;
+      const uint8_t* cur_b = lds + b_rd_base + sb * STAGE_B;
+      sa = (sa + 1 == kStagesA) ? 0 : sa + 1;
+      sb = (sb + 1 == kStagesB) ? 0 : sb + 1;
+      const uint8_t* nxt_a = lds + a_rd_base + sa * STAGE_A;
+      const uint8_t* nxt_b = lds + b_rd_base + sb * STAGE_B;
+
+      // [A] MFMAs on x* (first K half of this step) with the LDS reads of the second half
+      //     (-> y*) slotted one behind each; the reads sit in the front of the half step so
+      //     they have returned when the barrier wait needs them all. The fences pin this
+      //     interleaving: every wave-level memory instruction hides behind an MFMA.
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int t = 0; t < NMFMA; ++t) {
+        mfma_one(xa, xb, t);
+        if (t < NREAD) read_one(ya, yb, cur_a, cur_b, 1, t);
+        __builtin_amdgcn_sched_barrier(0);
+      }
+
+      // own loads of A(g+1) and B(g+1) have landed (B(g+2) may still be in flight); past the
+      // barrier everyone's have, and every wave is done reading this step's stages
+      if (KTAIL) wait_loads_and_barrier<0>();
+      else wait_loads_and_barrier<B_GROUPS>();
+
+      // [B] MFMAs on y* (second K half); behind each: one global->LDS load of A(g+2) / B(g+3)
+      //     into the stages just released (one load per MFMA keeps the wave from stalling on a
+      //     full load queue with the matrix pipe idle) and one LDS read of step g+1's first
+      //     half (-> x*; at the end of a tile these already belong to the next tile)
+      __builtin_amdgcn_sched_barrier(0);
+      if (!KTAIL) {
+        const uint8_t* ga = l_a + (size_t)ca.kt * kStepK;
+        const uint8_t* gb = l_b + (size_t)cb.kt * kStepK;
+        uint8_t* wa = lds + (ca.issued % kStagesA) * STAGE_A + wave * 1024;
+        uint8_t* wb = lds + LDS_B0 + (cb.issued % kStagesB) * STAGE_B + wave * 1024;
+        ++ca.issued;
+        ++cb.issued;
+#pragma unroll
+        for (int t = 0; t < NMFMA; ++t) {
+          mfma_one(ya, yb, t);
+          if (t < A_GROUPS) load_chunk_to_lds(ga + a_off[t], wa + NW * t * 1024);
+          else if (t < NLOAD) load_chunk_to_lds(gb + b_off[t - A_GROUPS], wb + NW * (t - A_GROUPS) * 1024);
+          if (t < NREAD) read_one(xa, xb, nxt_a, nxt_b, 0, t);
+          __builtin_amdgcn_sched_barrier(0);
+        }
+      } else {
+        issue_a();
+        issue_b();
+#pragma unroll
+        for (int t = 0; t < NMFMA; ++t) {
+          mfma_one(ya, yb, t);
+          if (t < NREAD) read_one(xa, xb, nxt_a, nxt_b, 0, t);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+      }
+      advance_a();
+      advance_b();
+    }
+    {
+      int tm, tn;
+      tile_coords(walk.chunk_begin + c_tile, p.tiles_m, p.tiles_n, p.group_m, tm, tn);
+      const int m0 = tm * BM, n0 = tn * BN;
+      const bool interior = (m0 + BM <= p.M) && (n0 + BN <= p.N) && ((p.ldc & 3) == 0) &&
+                            ((reinterpret_cast<uintptr_t>(p.c) & 7) == 0);
+      if (interior) epilogue(m0, n0, std::true_type{});
+      else epilogue(m0, n0, std::false_type{});
     }
   }
+  __builtin_amdgcn_s_waitcnt(0x0070);  // the trailing dummy loads must land before LDS is released
 }
 
 // ------------------------------------------------------------------------------------
@@ -501,16 +688,16 @@ int check_shape(int64_t M, int64_t N, int64_t K) {
   return MI355X_FP8_OK;
 }
 
-template <int BM, int BN, int WAVES_M, int WAVES_N, int SWZ_SHIFT>
+template <int BM, int BN, int WAVES_M, int WAVES_N, bool KTAIL, bool HAS_BIAS>
 int launch_tiled(GemmParams p, hipStream_t stream) {
   constexpr int threads = WAVES_M * WAVES_N * 64;
-  constexpr size_t lds_bytes = 2 * (size_t)(BM + BN) * kBK;
+  constexpr size_t lds_bytes = (size_t)(kStagesA * BM + kStagesB * BN) * kStepK;
   p.tiles_m = (p.M + BM - 1) / BM;
   p.tiles_n = (p.N + BN - 1) / BN;
   p.group_m = 4;
   const long total = (long)p.tiles_m * p.tiles_n;
   long grid = total < kNumCu ? ((total + kNumXcd - 1) / kNumXcd) * kNumXcd : kNumCu;
-  auto kern = gemm_tiled_kernel<BM, BN, WAVES_M, WAVES_N, SWZ_SHIFT>;
+  auto kern = gemm_tiled_kernel<BM, BN, WAVES_M, WAVES_N, KTAIL, HAS_BIAS>;
   static bool attr_set = false;  // raising the dynamic LDS limit is idempotent; races are harmless
   if (!attr_set) {
     hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize,
@@ -588,7 +775,8 @@ int mi355x_fp8_rowwise_gemm(const void* a, const void* b, const float* a_scale, 
       // b_scale is read 16 bytes at a time on full tiles
       if (reinterpret_cast<uintptr_t>(b_scale) & 15 || (bias && (reinterpret_cast<uintptr_t>(bias) & 7)))
         return fail(MI355X_FP8_ENOTSUP, "tiled variant needs b_scale 16-byte and bias 8-byte aligned");
-      return launch_tiled<256, 256, 2, 2, 0>(p, s);
+      if (K % kStepK) return bias ? launch_tiled<256, 256, 2, 2, true, true>(p, s) : launch_tiled<256, 256, 2, 2, true, false>(p, s);
+      return bias ? launch_tiled<256, 256, 2, 2, false, true>(p, s) : launch_tiled<256, 256, 2, 2, false, false>(p, s);
     case MI355X_FP8_VARIANT_SKINNY:
       if (M <= 16) return launch_skinny<1>(p, s);
       if (M <= 32) return launch_skinny<2>(p, s);
