@@ -154,10 +154,11 @@ struct StepCursor {
 // The kernel is one software pipeline over "steps" (a 128-byte K slab of one tile) that runs
 // through all tiles a workgroup owns without draining at tile boundaries. For step g:
 //
-//   [A] LDS reads of (g, second K half) interleaved with the MFMAs of (g, first K half)
+//   [A] MFMAs of (g, first K half), interleaved with the LDS reads of (g, second half) and
+//       the loads of B(g+2) (its stage was released at the previous barrier)
 //       wait for own loads of A(g+1) and B(g+1); workgroup barrier
-//   [B] issue loads A(g+2) and B(g+3) into the stages step g just released;
-//       LDS reads of (g+1, first half) interleaved with the MFMAs of (g, second half)
+//   [B] MFMAs of (g, second half), interleaved with the LDS reads of (g+1, first half) and
+//       the loads of A(g+2) into the A stage step g just released
 //   after a tile's last step: epilogue (loads of the next tile are already in flight)
 //
 // Two register sets of operand fragments alternate between the halves; one barrier per step.
@@ -326,18 +327,17 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_tiled_kernel(GemmP
     }
   };
   constexpr int NMFMA = MT * NT, NREAD = 2 * (MT + NT), NLOAD = A_GROUPS + B_GROUPS;
-  static_assert(NREAD <= NMFMA && NLOAD <= NMFMA, "one read and one load slot per MFMA");
+  static_assert(NREAD <= NMFMA && 2 * A_GROUPS <= NMFMA && 2 * B_GROUPS <= NMFMA, "one read slot per MFMA, one load slot per two");
 
-  // ---- prologue: A(0) B(0) A(1) B(1) B(2) in flight, first fragments in registers
+  // ---- prologue: A(0) B(0) A(1) B(1) in flight, first fragments in registers
   setup_a(ca.tile);
   setup_b(cb.tile);
   issue_a(); advance_a();
   issue_b(); advance_b();
   issue_a(); advance_a();
   issue_b(); advance_b();
-  issue_b(); advance_b();
   if (KTAIL) wait_loads_and_barrier<0>();
-  else wait_loads_and_barrier<A_GROUPS + 2 * B_GROUPS>();
+  else wait_loads_and_barrier<A_GROUPS + B_GROUPS>();
 #pragma unroll
   for (int u = 0; u < NREAD; ++u) read_one(xa, xb, lds + a_rd_base, lds + b_rd_base, 0, u);
 
@@ -420,46 +420,56 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_tiled_kernel(GemmP
       const uint8_t* nxt_a = lds + a_rd_base + sa * STAGE_A;
       const uint8_t* nxt_b = lds + b_rd_base + sb * STAGE_B;
 
-      // [A] MFMAs on x* (first K half of this step) with the LDS reads of the second half
-      //     (-> y*) slotted one behind each; the reads sit in the front of the half step so
-      //     they have returned when the barrier wait needs them all. The fences pin this
-      //     interleaving: every wave-level memory instruction hides behind an MFMA.
+      // [A] MFMAs on x* (first K half of this step). Behind them, one per MFMA: the LDS reads
+      //     of the second half (-> y*), and behind every other one a global->LDS load of
+      //     B(g+2) into the B stage released at the previous barrier. The fences pin this
+      //     interleaving: every wave-level memory instruction hides behind an MFMA, and the
+      //     load queue never holds more than the matrix pipe can cover.
       __builtin_amdgcn_sched_barrier(0);
+      if (!KTAIL) {
+        const uint8_t* gb = l_b + (size_t)cb.kt * kStepK;
+        uint8_t* wb = lds + LDS_B0 + (cb.issued % kStagesB) * STAGE_B + wave * 1024;
+        ++cb.issued;
 #pragma unroll
-      for (int t = 0; t < NMFMA; ++t) {
-        mfma_one(xa, xb, t);
-        if (t < NREAD) read_one(ya, yb, cur_a, cur_b, 1, t);
+        for (int t = 0; t < NMFMA; ++t) {
+          mfma_one(xa, xb, t);
+          if ((t & 1) == 0 && t / 2 < B_GROUPS) load_chunk_to_lds(gb + b_off[t / 2], wb + NW * (t / 2) * 1024);
+          if (t < NREAD) read_one(ya, yb, cur_a, cur_b, 1, t);
+          __builtin_amdgcn_sched_barrier(0);
+        }
+      } else {
+        issue_b();
+#pragma unroll
+        for (int t = 0; t < NMFMA; ++t) {
+          mfma_one(xa, xb, t);
+          if (t < NREAD) read_one(ya, yb, cur_a, cur_b, 1, t);
+        }
         __builtin_amdgcn_sched_barrier(0);
       }
+      advance_b();
 
       // own loads of A(g+1) and B(g+1) have landed (B(g+2) may still be in flight); past the
       // barrier everyone's have, and every wave is done reading this step's stages
       if (KTAIL) wait_loads_and_barrier<0>();
       else wait_loads_and_barrier<B_GROUPS>();
 
-      // [B] MFMAs on y* (second K half); behind each: one global->LDS load of A(g+2) / B(g+3)
-      //     into the stages just released (one load per MFMA keeps the wave from stalling on a
-      //     full load queue with the matrix pipe idle) and one LDS read of step g+1's first
-      //     half (-> x*; at the end of a tile these already belong to the next tile)
+      // [B] MFMAs on y* (second K half); behind them the loads of A(g+2) into the A stage just
+      //     released and the LDS reads of step g+1's first half (-> x*; at the end of a tile
+      //     these already belong to the next tile)
       __builtin_amdgcn_sched_barrier(0);
       if (!KTAIL) {
         const uint8_t* ga = l_a + (size_t)ca.kt * kStepK;
-        const uint8_t* gb = l_b + (size_t)cb.kt * kStepK;
         uint8_t* wa = lds + (ca.issued % kStagesA) * STAGE_A + wave * 1024;
-        uint8_t* wb = lds + LDS_B0 + (cb.issued % kStagesB) * STAGE_B + wave * 1024;
         ++ca.issued;
-        ++cb.issued;
 #pragma unroll
         for (int t = 0; t < NMFMA; ++t) {
           mfma_one(ya, yb, t);
-          if (t < A_GROUPS) load_chunk_to_lds(ga + a_off[t], wa + NW * t * 1024);
-          else if (t < NLOAD) load_chunk_to_lds(gb + b_off[t - A_GROUPS], wb + NW * (t - A_GROUPS) * 1024);
+          if ((t & 1) == 0 && t / 2 < A_GROUPS) load_chunk_to_lds(ga + a_off[t / 2], wa + NW * (t / 2) * 1024);
           if (t < NREAD) read_one(xa, xb, nxt_a, nxt_b, 0, t);
           __builtin_amdgcn_sched_barrier(0);
         }
       } else {
         issue_a();
-        issue_b();
 #pragma unroll
         for (int t = 0; t < NMFMA; ++t) {
           mfma_one(ya, yb, t);
@@ -468,7 +478,6 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_tiled_kernel(GemmP
         __builtin_amdgcn_sched_barrier(0);
       }
       advance_a();
-      advance_b();
     }
     {
       int tm, tn;
