@@ -493,112 +493,175 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_tiled_kernel(GemmP
 }
 
 // ------------------------------------------------------------------------------------
-// Skinny kernel (M <= 16*MT). Workgroup = KW waves sharing one 16-row panel of B; wave w
-// takes the 128-byte K steps w, w+KW, ... so that per iteration the workgroup reads one
-// contiguous KW*128-byte run of every row. Lane (r = lane%16, g = lane/16) loads, per
-// step, bytes [g*16, g*16+16) and [64+g*16, 64+g*16+16) of its row: each load
-// instruction then covers 64 contiguous bytes per row. A is read with the same mapping
-// straight from L2. Partial 16x16 tiles are summed across waves through LDS.
+// Skinny kernel (M <= 16*MT, HBM-bound): B is streamed exactly once and nothing is reused, so
+// what matters is whole-line coalesced loads and as many bytes in flight as a plain copy has.
+//
+// A workgroup owns 16*NTW rows of B and all of K; its 16 waves split K between them in
+// interleaved 128-byte steps (wave w takes steps w, w+16, ...: the workgroup reads 2 KB runs
+// of every row). Registers are the landing zone: a wave keeps DEPTH steps of loads in flight
+// (16 bytes per lane, 8 lanes per row, so every wave-wide load moves 8 whole 128-byte lines;
+// letting each MFMA lane fetch its own row instead costs the memory pipeline four times the
+// tag look-ups). A landed step is transposed into the MFMA lane layout through a small
+// wave-private LDS buffer (swizzled like the tiled kernel's stages); LDS executes a wave's
+// operations in order, so the loop needs no barrier. A [16*MT rows] takes the same route.
+// Partial 16x16 results are summed across the waves through LDS at the end.
 // ------------------------------------------------------------------------------------
-template <int MT, int KW>
+template <int MT, int NTW, int DEPTH, int KW>
 __global__ __launch_bounds__(KW * 64) void gemm_skinny_kernel(GemmParams p) {
-  __shared__ v4f red[KW][MT][64];
+  constexpr int TILE = 16 * kStepK;                 // one 16-row operand tile of one step: 2 KB
+  constexpr int NTILE = NTW + MT;                   // tiles per step: B tiles then A tiles
+  constexpr int LOADS = 2 * NTILE;                  // wave-wide loads per step
+  constexpr int BUF = NTILE * TILE;                 // wave-private transpose buffer
+  static_assert(NTW * MT * 1024 <= BUF, "the reduction reuses a wave's buffer for its partials");
+
+  extern __shared__ __attribute__((aligned(1024))) uint8_t lds[];
 
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-  const int r = lane & 15, g = lane >> 4;
-  const int n0 = blockIdx.x * 16;
+  uint8_t* buf = lds + wave * BUF;
+  const int n0 = blockIdx.x * (16 * NTW);
 
-  const uint8_t* bp = p.b + (size_t)min(n0 + r, p.N - 1) * p.ldb + g * kChunk;
-  const uint8_t* ap[MT];
+  // global load: lane (ld_row, ld_c) of a wave-wide load fetches chunk ld_c (16 bytes) of row
+  // ld_row of an 8-row half tile and parks it in LDS at the swizzled chunk position
+  const int ld_row = lane >> 3, ld_c = lane & 7;
+  const uint8_t* src[NTILE][2];
+  int wr_off[2];
 #pragma unroll
-  for (int t = 0; t < MT; ++t)
-    ap[t] = p.a + (size_t)min(t * 16 + r, p.M - 1) * p.lda + g * kChunk;
+  for (int h = 0; h < 2; ++h) {
+    const int r = h * 8 + ld_row;
+    wr_off[h] = r * kStepK + ((ld_c ^ swz128(r)) * kChunk);
+#pragma unroll
+    for (int t = 0; t < NTW; ++t)
+      src[t][h] = p.b + (size_t)min(n0 + t * 16 + r, p.N - 1) * p.ldb + ld_c * kChunk;
+#pragma unroll
+    for (int t = 0; t < MT; ++t)
+      src[NTW + t][h] = p.a + (size_t)min(t * 16 + r, p.M - 1) * p.lda + ld_c * kChunk;
+  }
+  // LDS->register: lane (r, g) of the 16x16x128 MFMA takes logical chunks 2g, 2g+1 of row r
+  const int r16 = lane & 15, g4 = lane >> 4;
+  const int rd0 = r16 * kStepK + (((2 * g4) ^ swz128(r16)) * kChunk);
+  const int rd1 = r16 * kStepK + (((2 * g4 + 1) ^ swz128(r16)) * kChunk);
 
-  v4f acc[MT];
-#pragma unroll
-  for (int t = 0; t < MT; ++t) acc[t] = (v4f){0.f, 0.f, 0.f, 0.f};
+  const int k_full = p.K / kStepK;
+  const int k_tail = p.K - k_full * kStepK;
+  const int my_steps = (k_full > wave) ? (k_full - wave + KW - 1) / KW : 0;  // whole steps this wave owns
 
-  const int k_full = p.K / kBK;
-  const int k_tail = p.K - k_full * kBK;
+  v4f acc[NTW][MT];
+#pragma unroll
+  for (int t = 0; t < NTW; ++t)
+#pragma unroll
+    for (int u = 0; u < MT; ++u) acc[t][u] = (v4f){0.f, 0.f, 0.f, 0.f};
 
-  constexpr int UNROLL = (MT == 1) ? 4 : 2;
-  int it = wave;
-  for (; it + (UNROLL - 1) * KW < k_full; it += UNROLL * KW) {
-    v4i b0[UNROLL], b1[UNROLL], a0[UNROLL][MT], a1[UNROLL][MT];
+  // DEPTH register sets, one per step in flight
+  v4i land[DEPTH][NTILE][2];
+  auto fetch = [&](int i, v4i (&dst)[NTILE][2]) {
+    const size_t kb = (size_t)(wave + KW * i) * kStepK;
 #pragma unroll
-    for (int u = 0; u < UNROLL; ++u) {
-      const size_t kb = (size_t)(it + u * KW) * kBK;
-      b0[u] = __builtin_nontemporal_load((const v4i*)(bp + kb));
-      b1[u] = __builtin_nontemporal_load((const v4i*)(bp + kb + 64));
-    }
+    for (int t = 0; t < NTILE; ++t)
 #pragma unroll
-    for (int u = 0; u < UNROLL; ++u) {
-      const size_t kb = (size_t)(it + u * KW) * kBK;
-#pragma unroll
-      for (int t = 0; t < MT; ++t) {
-        a0[u][t] = *(const v4i*)(ap[t] + kb);
-        a1[u][t] = *(const v4i*)(ap[t] + kb + 64);
+      for (int h = 0; h < 2; ++h) {
+        // B is read once and never again: stream it past the caches; A is shared by everyone
+        if (t < NTW) dst[t][h] = __builtin_nontemporal_load((const v4i*)(src[t][h] + kb));
+        else dst[t][h] = *(const v4i*)(src[t][h] + kb);
       }
+  };
+  auto consume = [&](const v4i (&got)[NTILE][2]) {
+#pragma unroll
+    for (int t = 0; t < NTILE; ++t)
+#pragma unroll
+      for (int h = 0; h < 2; ++h) *(v4i*)(buf + t * TILE + wr_off[h]) = got[t][h];
+    v8i f[NTILE];
+#pragma unroll
+    for (int t = 0; t < NTILE; ++t) {
+      const v4i lo = *(const v4i*)(buf + t * TILE + rd0);
+      const v4i hi = *(const v4i*)(buf + t * TILE + rd1);
+      f[t] = (v8i){lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
     }
 #pragma unroll
-    for (int u = 0; u < UNROLL; ++u) {
-      const v8i bf = {b0[u][0], b0[u][1], b0[u][2], b0[u][3], b1[u][0], b1[u][1], b1[u][2], b1[u][3]};
+    for (int t = 0; t < NTW; ++t)
 #pragma unroll
-      for (int t = 0; t < MT; ++t) {
-        const v8i af = {a0[u][t][0], a0[u][t][1], a0[u][t][2], a0[u][t][3],
-                        a1[u][t][0], a1[u][t][1], a1[u][t][2], a1[u][t][3]};
-        acc[t] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(bf, af, acc[t], 0, 0, 0, 0, 0, 0);
+      for (int u = 0; u < MT; ++u)
+        acc[t][u] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(f[t], f[NTW + u], acc[t][u], 0, 0, 0, 0, 0, 0);
+  };
+
+  // The loop is unrolled DEPTH times so every register set has a fixed name; the compiler's
+  // own wait counts make each consume() wait for exactly its set's loads (they return in
+  // issue order, so the younger sets stay in flight).
+#pragma unroll
+  for (int d = 0; d < DEPTH; ++d)
+    if (d < my_steps) fetch(d, land[d]);
+  for (int i = 0; i < my_steps; i += DEPTH) {
+#pragma unroll
+    for (int d = 0; d < DEPTH; ++d) {
+      if (i + d < my_steps) {
+        consume(land[d]);
+        if (i + d + DEPTH < my_steps) fetch(i + d + DEPTH, land[d]);
       }
     }
   }
-  // leftover whole steps, then the partial step (taken by the wave whose turn it is)
-  for (; it < k_full + (k_tail ? 1 : 0); it += KW) {
-    const size_t kb = (size_t)it * kBK;
-    const int lim = (it < k_full) ? kBK : k_tail;
-    const bool in0 = g * kChunk < lim, in1 = 64 + g * kChunk < lim;
+  // K tail (K % 128 != 0): one partial step, taken by the wave whose turn it would be; the
+  // lanes fetch their own 16-byte chunks and chunks at or past K count as zero
+  if (k_tail && (k_full % KW) == wave) {
+    const size_t kb = (size_t)k_full * kStepK;
+    const bool in0 = (2 * g4) * kChunk < k_tail, in1 = (2 * g4 + 1) * kChunk < k_tail;
     const v4i z = {0, 0, 0, 0};
-    const v4i b0 = in0 ? *(const v4i*)(bp + kb) : z;
-    const v4i b1 = in1 ? *(const v4i*)(bp + kb + 64) : z;
-    const v8i bf = {b0[0], b0[1], b0[2], b0[3], b1[0], b1[1], b1[2], b1[3]};
+    v8i bf[NTW], af[MT];
 #pragma unroll
-    for (int t = 0; t < MT; ++t) {
-      const v4i a0 = in0 ? *(const v4i*)(ap[t] + kb) : z;
-      const v4i a1 = in1 ? *(const v4i*)(ap[t] + kb + 64) : z;
-      const v8i af = {a0[0], a0[1], a0[2], a0[3], a1[0], a1[1], a1[2], a1[3]};
-      acc[t] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(bf, af, acc[t], 0, 0, 0, 0, 0, 0);
+    for (int t = 0; t < NTW; ++t) {
+      const uint8_t* row = p.b + (size_t)min(n0 + t * 16 + r16, p.N - 1) * p.ldb + kb;
+      const v4i lo = in0 ? *(const v4i*)(row + 2 * g4 * kChunk) : z;
+      const v4i hi = in1 ? *(const v4i*)(row + (2 * g4 + 1) * kChunk) : z;
+      bf[t] = (v8i){lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
     }
+#pragma unroll
+    for (int u = 0; u < MT; ++u) {
+      const uint8_t* row = p.a + (size_t)min(u * 16 + r16, p.M - 1) * p.lda + kb;
+      const v4i lo = in0 ? *(const v4i*)(row + 2 * g4 * kChunk) : z;
+      const v4i hi = in1 ? *(const v4i*)(row + (2 * g4 + 1) * kChunk) : z;
+      af[u] = (v8i){lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+    }
+#pragma unroll
+    for (int t = 0; t < NTW; ++t)
+#pragma unroll
+      for (int u = 0; u < MT; ++u)
+        acc[t][u] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(bf[t], af[u], acc[t][u], 0, 0, 0, 0, 0, 0);
   }
 
+  // ---- cross-wave reduction through each wave's own (now idle) buffer
+  v4f* mine = (v4f*)buf;
 #pragma unroll
-  for (int t = 0; t < MT; ++t) red[wave][t][lane] = acc[t];
+  for (int t = 0; t < NTW; ++t)
+#pragma unroll
+    for (int u = 0; u < MT; ++u) mine[(t * MT + u) * 64 + lane] = acc[t][u];
   __syncthreads();
 
-  // Lane layout of a 16x16 result: m = t*16 + lane%16, n = n0 + 4*(lane/16) + e.
-  for (int idx = threadIdx.x; idx < MT * 64; idx += KW * 64) {
-    const int t = idx >> 6, l = idx & 63;
-    v4f s = red[0][t][l];
+  // Lane layout of a 16x16 result: m = u*16 + lane%16, n = n0 + t*16 + 4*(lane/16) + e.
+  for (int idx = threadIdx.x; idx < NTW * MT * 64; idx += KW * 64) {
+    const int tu = idx >> 6, l = idx & 63;
+    const int t = tu / MT, u = tu % MT;
+    v4f sum = ((const v4f*)lds)[tu * 64 + l];
 #pragma unroll
-    for (int w = 1; w < KW; ++w) s += red[w][t][l];
-    const int m = t * 16 + (l & 15);
-    const int n = n0 + 4 * (l >> 4);
-    if (m >= p.M) continue;
+    for (int w = 1; w < KW; ++w) sum += ((const v4f*)(lds + w * BUF))[tu * 64 + l];
+    const int m = u * 16 + (l & 15);
+    const int n = n0 + t * 16 + 4 * (l >> 4);
+    if (m >= p.M || n >= p.N) continue;
     const float sa_m = p.a_scale[m];
-    uint16_t* crow = p.c + (size_t)m * p.ldc;
-    uint16_t o[4];
+    float r[4];
 #pragma unroll
     for (int e = 0; e < 4; ++e) {
       const int ne = min(n + e, p.N - 1);
-      float v = s[e] * sa_m * p.b_scale[ne];
-      if (p.bias) v += bf16_to_f32(p.bias[ne]);
-      o[e] = f32_to_bf16_rne(v);
+      r[e] = sum[e] * sa_m * p.b_scale[ne];
+      if (p.bias) r[e] += bf16_to_f32(p.bias[ne]);
     }
+    const uint32_t lo = pack_bf16x2(r[0], r[1]), hi = pack_bf16x2(r[2], r[3]);
+    uint16_t* dst = p.c + (size_t)m * p.ldc + n;
     if (n + 3 < p.N && ((p.ldc & 3) == 0) && ((reinterpret_cast<uintptr_t>(p.c) & 7) == 0)) {
-      *(us4*)(crow + n) = (us4){o[0], o[1], o[2], o[3]};
+      *(v2u*)dst = (v2u){lo, hi};
     } else {
-#pragma unroll
-      for (int e = 0; e < 4; ++e)
-        if (n + e < p.N) crow[n + e] = o[e];
+      dst[0] = (uint16_t)lo;
+      if (n + 1 < p.N) dst[1] = (uint16_t)(lo >> 16);
+      if (n + 2 < p.N) dst[2] = (uint16_t)hi;
+      if (n + 3 < p.N) dst[3] = (uint16_t)(hi >> 16);
     }
   }
 }
@@ -720,11 +783,19 @@ int launch_tiled(GemmParams p, hipStream_t stream) {
   return MI355X_FP8_OK;
 }
 
-template <int MT>
+template <int MT, int NTW, int DEPTH, int KW>
 int launch_skinny(const GemmParams& p, hipStream_t stream) {
-  constexpr int KW = 8;
-  const unsigned grid = (unsigned)((p.N + 15) / 16);
-  hipLaunchKernelGGL((gemm_skinny_kernel<MT, KW>), dim3(grid), dim3(KW * 64), 0, stream, p);
+  constexpr size_t lds_bytes = (size_t)KW * (NTW + MT) * 16 * kStepK;
+  static_assert(lds_bytes <= 160 * 1024, "transpose buffers must fit the 160 KB LDS");
+  auto kern = gemm_skinny_kernel<MT, NTW, DEPTH, KW>;
+  static bool attr_set = false;
+  if (!attr_set) {
+    hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
+    if (e != hipSuccess) return fail(MI355X_FP8_ELAUNCH, "hipFuncSetAttribute: %s", hipGetErrorString(e));
+    attr_set = true;
+  }
+  const unsigned grid = (unsigned)((p.N + 16 * NTW - 1) / (16 * NTW));
+  hipLaunchKernelGGL(kern, dim3(grid), dim3(KW * 64), lds_bytes, stream, p);
   hipError_t e = hipGetLastError();
   if (e != hipSuccess) return fail(MI355X_FP8_ELAUNCH, "skinny kernel launch: %s", hipGetErrorString(e));
   return MI355X_FP8_OK;
@@ -787,10 +858,14 @@ int mi355x_fp8_rowwise_gemm(const void* a, const void* b, const float* a_scale, 
       if (K % kStepK) return bias ? launch_tiled<256, 256, 2, 2, true, true>(p, s) : launch_tiled<256, 256, 2, 2, true, false>(p, s);
       return bias ? launch_tiled<256, 256, 2, 2, false, true>(p, s) : launch_tiled<256, 256, 2, 2, false, false>(p, s);
     case MI355X_FP8_VARIANT_SKINNY:
-      if (M <= 16) return launch_skinny<1>(p, s);
-      if (M <= 32) return launch_skinny<2>(p, s);
-      if (M <= 48) return launch_skinny<3>(p, s);
-      return launch_skinny<4>(p, s);
+      // 16-row blocks of A | B tiles per wave | steps in flight per wave (sized to 128 VGPRs)
+#ifndef SKCFG
+#define SKCFG 1, 1, 4, 8
+#endif
+      if (M <= 16) return launch_skinny<SKCFG>(p, s);
+      if (M <= 32) return launch_skinny<2, 1, 2, 8>(p, s);
+      if (M <= 48) return launch_skinny<3, 1, 2, 8>(p, s);
+      return launch_skinny<4, 1, 2, 8>(p, s);
     default:
       return fail(MI355X_FP8_EINVAL, "unknown variant %d", variant);
   }
