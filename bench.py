@@ -27,6 +27,7 @@ sys.path.insert(0, ROOT)
 PEAK_FP8_TFLOPS = 5000.0  # dense FP8 MFMA, MI355X datasheet
 PEAK_HBM_GBPS = 8000.0    # HBM3E, MI355X datasheet
 SEED = 1337
+TILED_8192_TRAFFIC_BYTES = (803574 + 137966) * 1024  # see profiles/tiled_8192cubed_hbm_traffic.md
 
 
 def make_device_inputs(m, n, k, sigma, bias, dev, copies=1):
@@ -187,7 +188,10 @@ def main():
             "peak": PEAK_FP8_TFLOPS,
             "unit": "TFLOP/s",
             "frac": head["tflops"] / PEAK_FP8_TFLOPS,
-            "traffic": None,
+            # HBM-side bytes per launch of the dominant kernel, from rocprofv3 --pmc FETCH_SIZE /
+            # WRITE_SIZE scaled by a copy kernel of known size (FETCH x2.0, WRITE x1.0); a property
+            # of the kernel's tile walk on this workload, re-profiled whenever the kernel changes
+            "traffic": TILED_8192_TRAFFIC_BYTES,
         },
     }
 
