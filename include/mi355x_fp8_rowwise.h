@@ -51,6 +51,20 @@ extern "C" {
 #define MI355X_FP8_VARIANT_TILED   1  /* LDS-tiled persistent MFMA kernel (compute-bound shapes) */
 #define MI355X_FP8_VARIANT_SKINNY  2  /* in-workgroup split-K streaming kernel (M <= 64, HBM-bound) */
 
+/*
+ * The `variant` argument is a word: bits 0..7 hold the family above; for the tiled family
+ * bits 8..15 may pin the tile configuration and bits 16..23 the split-K factor (0 in a
+ * field = chosen by the library from the shape). Tile configurations: 0 = 256x256 tiles,
+ * one workgroup per CU; 1 = 128x128 tiles, two workgroups per CU. With a split-K factor
+ * S > 1 every tile's K range is cut into S parts that run as separate work items; they
+ * leave fp32 partial sums in the workspace (S*M*N*4 bytes) and a second kernel adds them
+ * in a fixed order, so results do not depend on scheduling. A split factor larger than the
+ * number of 128-byte K steps is reduced to it.
+ */
+#define MI355X_FP8_TILED_CONFIG(cfg)    ((((cfg) + 1) & 0xff) << 8)
+#define MI355X_FP8_TILED_SPLITS(s)      (((s) & 0xff) << 16)
+#define MI355X_FP8_NUM_TILE_CONFIGS     2
+
 /* Source element types accepted by the quantiser. */
 #define MI355X_FP8_SRC_F32   0
 #define MI355X_FP8_SRC_BF16  1
@@ -63,7 +77,8 @@ const char* mi355x_fp8_rowwise_last_error(void);
  * or a negative status when the shape is not supported. Lets tests pin the dispatch. */
 int mi355x_fp8_rowwise_select_variant(int64_t M, int64_t N, int64_t K);
 
-/* Bytes of device workspace `variant` needs for this shape (0 when none). */
+/* Bytes of device workspace `variant` needs for this shape (0 when none). Pure host
+ * arithmetic: callable without a device. */
 size_t mi355x_fp8_rowwise_workspace_bytes(int64_t M, int64_t N, int64_t K, int variant);
 
 /*
@@ -77,7 +92,10 @@ size_t mi355x_fp8_rowwise_workspace_bytes(int64_t M, int64_t N, int64_t K, int v
  *   bias     bf16 [N] or NULL                   c        bf16 [M, N], row stride ldc
  *
  * Requirements: M, N, K >= 1; K, lda, ldb multiples of 16; a and b 16-byte aligned.
- * `workspace` may be NULL when mi355x_fp8_rowwise_workspace_bytes() is 0.
+ * `workspace` (16-byte aligned) may be NULL when mi355x_fp8_rowwise_workspace_bytes() is 0.
+ * A call whose variant leaves the split-K factor to the library and brings less workspace
+ * than that runs the best plan that needs none (same results up to fp32 summation order);
+ * a call that names a split factor > 1 without enough workspace fails with EINVAL.
  */
 int mi355x_fp8_rowwise_gemm(const void* a, const void* b,
                             const float* a_scale, const float* b_scale,

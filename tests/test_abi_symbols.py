@@ -60,3 +60,26 @@ def test_status_to_exception_mapping():
     with pytest.raises(ValueError):
         _lib.check(lib.mi355x_fp8_rowwise_select_variant(-1, 8, 16), "select")
     _lib.check(0, "fine")
+
+
+def test_workspace_size_follows_the_plan_without_a_gpu():
+    lib = _lib.load()
+    ws = lib.mi355x_fp8_rowwise_workspace_bytes
+    text = open(HEADER).read()
+    assert int(re.search(r"#define\s+MI355X_FP8_NUM_TILE_CONFIGS\s+(\d+)", text).group(1)) == _lib.NUM_TILE_CONFIGS
+    # enough tiles to fill the chip, or the on-chip reduction of the skinny kernel: no workspace
+    assert ws(8192, 8192, 8192, _lib.VARIANT_AUTO) == 0
+    assert ws(16, 8192, 8192, _lib.VARIANT_AUTO) == 0
+    assert ws(16, 8192, 8192, _lib.VARIANT_SKINNY) == 0
+    # few tiles and a long K: split, S * M * N fp32 partial sums
+    auto = ws(128, 8192, 8192, _lib.VARIANT_AUTO)
+    assert auto > 0 and auto % (128 * 8192 * 4) == 0
+    # a pinned split factor is honoured, clipped to the number of 128-byte K steps
+    assert ws(256, 256, 1024, _lib.tiled_variant(0, 4)) == 4 * 256 * 256 * 4
+    assert ws(256, 256, 1024, _lib.tiled_variant(1, 1)) == 0
+    assert ws(256, 256, 256, _lib.tiled_variant(0, 16)) == 2 * 256 * 256 * 4
+    assert ws(256, 256, 128, _lib.tiled_variant(0, 16)) == 0
+    # 9 steps in 4 parts of 3: only 3 parts are non-empty
+    assert ws(256, 256, 9 * 128, _lib.tiled_variant(0, 4)) == 3 * 256 * 256 * 4
+    # unsupported shapes need nothing (the GEMM call itself reports the error)
+    assert ws(8, 8, 24, _lib.VARIANT_AUTO) == 0

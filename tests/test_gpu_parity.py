@@ -93,6 +93,83 @@ def test_seeded_shapes_against_oracle(gpu_device, m, n, k, bias, variant):
     _check_tight(out, xq, wq, xs, ws, b)
 
 
+PLAN_SHAPES = [
+    # m, n, k, bias: ragged edges in both tile sizes, K tails, K shorter than the split count
+    (130, 260, 128, True), (257, 129, 1040, False), (300, 520, 2048, True), (127, 1000, 4112, True),
+    (512, 384, 640, False),
+]
+
+
+@pytest.mark.parametrize("m,n,k,bias", PLAN_SHAPES)
+@pytest.mark.parametrize("config", range(_lib.NUM_TILE_CONFIGS))
+@pytest.mark.parametrize("splits", [1, 2, 3, 5, 16])
+def test_every_tile_config_and_split_factor(gpu_device, m, n, k, bias, config, splits):
+    print(f"case m={m} n={n} k={k} bias={bias} config={config} splits={splits}", flush=True)
+    xq, wq, xs, ws, b = orc.make_inputs(m, n, k, 1.0, bias)
+    want = orc.dequant_matmul(xq, wq, xs, ws, b)
+    out = _run(gpu_device, xq, wq, xs, ws, b, _lib.tiled_variant(config, splits))
+    torch.testing.assert_close(out, want, rtol=RTOL, atol=ATOL)
+    _check_tight(out, xq, wq, xs, ws, b)
+
+
+@pytest.mark.parametrize("config", range(_lib.NUM_TILE_CONFIGS))
+def test_split_k_exact_integer_case_is_bit_exact(gpu_device, config):
+    # as test_exact_integer_case_is_bit_exact, with the sum cut into 4 partial sums that meet
+    # in the finalize kernel; the output sits inside a larger buffer guarded by canaries
+    rng = np.random.default_rng(12)
+    ints = np.array([0, 1, 2, 3, 4, -1, -2, -3, -4, 0.5, -0.5], dtype=np.float32)
+    m, n, k = 200, 391, 1296
+    a = rng.choice(ints, size=(m, k)).astype(np.float32)
+    b = rng.choice(ints, size=(n, k)).astype(np.float32)
+    dev = gpu_device
+    c_buf = torch.full((m + 2, n + 9), -77.0, dtype=torch.bfloat16, device=dev)
+    c_view = c_buf[1:m + 1, 3:3 + n]
+    ops.fp8_gemm_rowwise(torch.from_numpy(a).to(torch.float8_e4m3fn).to(dev), torch.from_numpy(b).to(torch.float8_e4m3fn).to(dev),
+                         torch.ones(m, device=dev), torch.ones(n, device=dev), out=c_view,
+                         variant=_lib.tiled_variant(config, 4))
+    torch.cuda.synchronize()
+    want = orc.to_bf16_bits((a.astype(np.float64) @ b.astype(np.float64).T).astype(np.float32))
+    assert np.array_equal(_bits(c_view.contiguous()), want)
+    mask = torch.ones_like(c_buf, dtype=torch.bool)
+    mask[1:m + 1, 3:3 + n] = False
+    assert torch.all(c_buf[mask] == -77.0)
+
+
+def test_workspace_rules(gpu_device):
+    dev = gpu_device
+    lib = _lib.load()
+    m, n, k = 128, 2048, 8192
+    xq, wq, xs, ws, _ = orc.make_inputs(m, n, k, 1.0, False)
+    dxq, dwq, dxs, dws = (t.to(dev) for t in (xq, wq, xs, ws))
+    want = orc.dequant_matmul(xq, wq, xs, ws, None)
+    auto = _lib.VARIANT_AUTO
+    need = lib.mi355x_fp8_rowwise_workspace_bytes(m, n, k, auto)
+    assert need > 0 and need % (m * n * 4) == 0  # few tiles, long K: the library splits K
+    out = torch.empty((m, n), dtype=torch.bfloat16, device=dev)
+
+    def call(variant, wsp, wsp_bytes):
+        return lib.mi355x_fp8_rowwise_gemm(dxq.data_ptr(), dwq.data_ptr(), dxs.data_ptr(), dws.data_ptr(), None,
+                                           out.data_ptr(), m, n, k, k, k, n, wsp, wsp_bytes, variant,
+                                           torch.cuda.current_stream().cuda_stream)
+
+    # automatic plan without workspace: runs a plan that needs none
+    out.fill_(-3.0)
+    assert call(auto, None, 0) == _lib.OK
+    torch.cuda.synchronize()
+    torch.testing.assert_close(out.cpu(), want, rtol=RTOL, atol=ATOL)
+    # pinned split factor without enough workspace: refused, nothing launched
+    buf = torch.empty(need, dtype=torch.uint8, device=dev)
+    out.fill_(-3.0)
+    assert call(_lib.tiled_variant(None, 4), buf.data_ptr(), m * n * 4) == _lib.EINVAL
+    assert b"workspace" in lib.mi355x_fp8_rowwise_last_error()
+    torch.cuda.synchronize()
+    assert torch.all(out == -3.0)
+    # with the workspace: the split plan
+    assert call(auto, buf.data_ptr(), need) == _lib.OK
+    torch.cuda.synchronize()
+    torch.testing.assert_close(out.cpu(), want, rtol=RTOL, atol=ATOL)
+
+
 @pytest.mark.parametrize("m", [1, 2, 15, 16, 17, 31, 32, 33, 47, 48, 49, 63, 64])
 def test_skinny_every_row_count(gpu_device, m):
     n, k = 1000, 1168
@@ -225,6 +302,9 @@ def test_unsupported_and_invalid_arguments_raise(gpu_device):
         ops.fp8_gemm_rowwise(f8(16, 16), f8(16, 16), torch.ones(15, device=dev), torch.ones(16, device=dev))
     with pytest.raises(ValueError, match="unknown variant"):
         ops.fp8_gemm_rowwise(f8(16, 16), f8(16, 16), torch.ones(16, device=dev), torch.ones(16, device=dev), variant=99)
+    with pytest.raises(ValueError, match="unknown variant"):
+        ops.fp8_gemm_rowwise(f8(16, 16), f8(16, 16), torch.ones(16, device=dev), torch.ones(16, device=dev),
+                             variant=_lib.tiled_variant(_lib.NUM_TILE_CONFIGS))
 
 
 def test_dispatch_is_pinned(gpu_device):
@@ -236,7 +316,7 @@ def test_dispatch_is_pinned(gpu_device):
 def test_graph_capture_replays_match_eager(gpu_device):
     # the benchmark harness times the callable inside a captured graph on a side stream
     dev = gpu_device
-    for (m, n, k) in [(16, 2048, 2048), (300, 512, 1040)]:
+    for (m, n, k) in [(16, 2048, 2048), (300, 512, 1040), (128, 1024, 8192)]:  # skinny, tiled, split-K
         xq, wq, xs, ws, b = orc.make_inputs(m, n, k, 1.0, True)
         dxq, dwq, dxs, dws, db = (t.to(dev) for t in (xq, wq, xs, ws, b))
         eager = ops.fp8_gemm_rowwise(dxq, dwq, dxs, dws, bias=db)

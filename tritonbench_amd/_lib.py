@@ -22,6 +22,18 @@ VARIANT_AUTO = 0
 VARIANT_TILED = 1
 VARIANT_SKINNY = 2
 
+NUM_TILE_CONFIGS = 2
+
+
+def tiled_variant(config=None, splits=0) -> int:
+    """Variant word of the tiled family with the tile configuration and/or split-K factor
+    pinned (MI355X_FP8_TILED_CONFIG / MI355X_FP8_TILED_SPLITS of the header)."""
+    word = VARIANT_TILED
+    if config is not None:
+        word |= ((config + 1) & 0xFF) << 8
+    return word | ((splits & 0xFF) << 16)
+
+
 SRC_F32 = 0
 SRC_BF16 = 1
 

@@ -50,6 +50,11 @@ struct GemmParams {
   long lda, ldb, ldc;
   int tiles_m, tiles_n;
   int group_m;           // tile rows walked together so an XCD's resident tiles share A and B panels
+  // split-K: every tile is cut into `splits` work items of `steps_per_split` 128-byte K steps
+  // (the last one takes what is left); with splits > 1 the items write fp32 partial sums to
+  // partial[split][M][N] and a second kernel adds them up and applies the epilogue
+  int splits, steps_per_split;
+  float* partial;
 };
 
 __device__ __forceinline__ uint16_t f32_to_bf16_rne(float f) {
@@ -128,6 +133,10 @@ __device__ __forceinline__ void load_chunk_to_lds(const uint8_t* gsrc, uint8_t* 
       (__attribute__((address_space(3))) void*)lds_wave_base, 16, 0, 0);
 }
 
+// Source of the chunks that lie past K in the last, partial K step: the operands there must
+// read as zeros (whatever follows a row in memory could decode to NaN).
+__device__ const v4i kZeroChunk = {0, 0, 0, 0};
+
 // Scheduling hints for the machine scheduler: MFMA / LDS read / global load slots.
 #define SCHED_MFMA(n) __builtin_amdgcn_sched_group_barrier(0x008, n, 0)
 #define SCHED_DSREAD(n) __builtin_amdgcn_sched_group_barrier(0x100, n, 0)
@@ -148,7 +157,7 @@ __device__ __forceinline__ void wait_loads_and_barrier() {
 // Cursor over the (tile, K step) sequence a workgroup walks; one for the A loads, one for
 // the B loads (which run a step further ahead).
 struct StepCursor {
-  int tile, kt, issued;
+  int item, kt, kt_end, issued;
 };
 
 // The kernel is one software pipeline over "steps" (a 128-byte K slab of one tile) that runs
@@ -162,8 +171,22 @@ struct StepCursor {
 //   after a tile's last step: epilogue (loads of the next tile are already in flight)
 //
 // Two register sets of operand fragments alternate between the halves; one barrier per step.
-template <int BM, int BN, int WAVES_M, int WAVES_N, bool KTAIL, bool HAS_BIAS>
-__global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_tiled_kernel(GemmParams p) {
+//
+// EPI selects what happens to a finished accumulator tile: scaled bf16 store (kEpiPlain),
+// the same with the bias added (kEpiBias), or a raw fp32 partial-sum store for split-K
+// (kEpiPartial). Tiles small enough for two workgroups per CU are compiled for two waves per
+// SIMD (256 registers each).
+constexpr int kEpiPlain = 0, kEpiBias = 1, kEpiPartial = 2;
+
+constexpr size_t tiled_lds_bytes(int BM, int BN) { return (size_t)(kStagesA * BM + kStagesB * BN) * kStepK; }
+constexpr int tiled_wgs_per_cu(int BM, int BN) { return tiled_lds_bytes(BM, BN) <= 80 * 1024 ? 2 : 1; }
+
+template <int BM, int BN, int WAVES_M, int WAVES_N, bool KTAIL, int EPI>
+__global__ __launch_bounds__(WAVES_M* WAVES_N * 64)
+__attribute__((amdgpu_waves_per_eu(tiled_wgs_per_cu(BM, BN) * WAVES_M * WAVES_N / 4,
+                                   tiled_wgs_per_cu(BM, BN) * WAVES_M * WAVES_N / 4)))
+void gemm_tiled_kernel(GemmParams p) {
+  constexpr bool HAS_BIAS = EPI == kEpiBias;
   constexpr int NW = WAVES_M * WAVES_N;
   constexpr int WTM = BM / WAVES_M;    // wave tile rows (m)
   constexpr int WTN = BN / WAVES_N;    // wave tile cols (n)
@@ -202,17 +225,24 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_tiled_kernel(GemmP
   const int a_rd_base = (wm * WTM) * kStepK;
   const int b_rd_base = LDS_B0 + (wn * WTN) * kStepK;
 
+  // Work items are (split, tile) pairs, split-major: consecutive items are neighbouring
+  // tiles of the same K range, so an XCD's chunk of the list still shares operand panels.
   const int total_tiles = p.tiles_m * p.tiles_n;
-  const TileWalk walk = make_walk(total_tiles);
+  const TileWalk walk = make_walk(total_tiles * p.splits);
   if (walk.slot >= walk.chunk_len) return;  // uniform over the workgroup
-  const int my_tiles = (walk.chunk_len - walk.slot + walk.slots - 1) / walk.slots;
   const int k_full = p.K / kStepK;             // whole 128-byte steps
   const int k_tail = p.K - k_full * kStepK;    // 0 or a multiple of 16
   const int k_steps = k_full + (k_tail ? 1 : 0);
-  const int total_steps = my_tiles * k_steps;
+  auto item_split = [&](int li) { return (walk.chunk_begin + li) / total_tiles; };
+  auto item_tile = [&](int li) { return (walk.chunk_begin + li) % total_tiles; };
+  auto split_begin = [&](int sp) { return sp * p.steps_per_split; };
+  auto split_end = [&](int sp) { return min((sp + 1) * p.steps_per_split, k_steps); };
+  int total_steps = 0;
+  for (int li = walk.slot; li < walk.chunk_len; li += walk.slots)
+    total_steps += split_end(item_split(li)) - split_begin(item_split(li));
 
   // ---- load side of the pipeline
-  StepCursor ca = {walk.slot, 0, 0}, cb = {walk.slot, 0, 0};
+  StepCursor ca = {walk.slot, 0, 0, 0}, cb = {walk.slot, 0, 0, 0};
   const uint8_t* l_a = nullptr;
   const uint8_t* l_b = nullptr;
   uint32_t a_off[A_GROUPS], b_off[B_GROUPS];
@@ -220,7 +250,9 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_tiled_kernel(GemmP
   // stored, so every load stays in bounds without predication.
   auto setup_a = [&](int li) {
     int tm, tn;
-    tile_coords(walk.chunk_begin + li, p.tiles_m, p.tiles_n, p.group_m, tm, tn);
+    tile_coords(item_tile(li), p.tiles_m, p.tiles_n, p.group_m, tm, tn);
+    ca.kt = split_begin(item_split(li));
+    ca.kt_end = split_end(item_split(li));
     const int m0 = tm * BM;
     l_a = p.a + (size_t)m0 * p.lda;
 #pragma unroll
@@ -231,7 +263,9 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_tiled_kernel(GemmP
   };
   auto setup_b = [&](int li) {
     int tm, tn;
-    tile_coords(walk.chunk_begin + li, p.tiles_m, p.tiles_n, p.group_m, tm, tn);
+    tile_coords(item_tile(li), p.tiles_m, p.tiles_n, p.group_m, tm, tn);
+    cb.kt = split_begin(item_split(li));
+    cb.kt_end = split_end(item_split(li));
     const int n0 = tn * BN;
     l_b = p.b + (size_t)n0 * p.ldb;
 #pragma unroll
@@ -243,25 +277,23 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_tiled_kernel(GemmP
   // Issues one operand's loads for its cursor's step into stage (issued % STAGES). Past the
   // last step it re-issues the last one into a stage nobody reads again, which keeps the
   // path free of branches.
+  // K tail (KTAIL kernels only): in the partial last step, lanes whose chunk lies at or past
+  // K fetch the zero chunk instead. A lane's logical chunk is the same for all its groups
+  // (the swizzle key depends on the group's parity only, and a wave's groups are NW apart).
+  static_assert(NW % 2 == 0, "all groups of a wave must share their parity");
+  const bool tail_chunk_ok = ((ld_pc ^ swz128(wave * 8 + ld_row)) * kChunk) < k_tail;
+  auto chunk_src = [&](const uint8_t* g, uint32_t off, bool real) -> const uint8_t* {
+    if (!KTAIL) return g + off;
+    return real ? g + off : reinterpret_cast<const uint8_t*>(&kZeroChunk);
+  };
+  constexpr int MAX_GROUPS = A_GROUPS > B_GROUPS ? A_GROUPS : B_GROUPS;
   auto issue = [&](const uint8_t* gbase, const uint32_t* off, int groups, int kt, uint8_t* sbase) {
     const uint8_t* g = gbase + (size_t)kt * kStepK;
-    if (!KTAIL || kt < k_full) {
+    const bool real = !KTAIL || kt < k_full || tail_chunk_ok;
 #pragma unroll
-      for (int i = 0; i < A_GROUPS; ++i)
-        if (i < groups) load_chunk_to_lds(g + off[i], sbase + (wave + NW * i) * 1024);
-    } else {
-      // K tail: chunks at or past K are written as zeros (they would pollute the sums)
-#pragma unroll
-      for (int i = 0; i < A_GROUPS; ++i) {
-        if (i >= groups) continue;
-        const int c = ld_pc ^ swz128((wave + NW * i) * 8 + ld_row);
-        v4i v = {0, 0, 0, 0};
-        if (c * kChunk < k_tail) v = *(const v4i*)(g + off[i]);
-        *(v4i*)(sbase + (wave + NW * i) * 1024 + lane * kChunk) = v;
-      }
-    }
+    for (int i = 0; i < MAX_GROUPS; ++i)
+      if (i < groups) load_chunk_to_lds(chunk_src(g, off[i], real), sbase + (wave + NW * i) * 1024);
   };
-  static_assert(A_GROUPS == B_GROUPS, "issue() unrolls over A_GROUPS for both operands");
   auto issue_a = [&]() {
     issue(l_a, a_off, A_GROUPS, ca.kt, lds + (ca.issued % kStagesA) * STAGE_A);
     ++ca.issued;
@@ -272,18 +304,16 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_tiled_kernel(GemmP
   };
   auto advance_a = [&]() {
     if (ca.issued >= total_steps) return;  // stay on the last step
-    if (++ca.kt == k_steps) {
-      ca.kt = 0;
-      ca.tile += walk.slots;
-      setup_a(ca.tile);
+    if (++ca.kt == ca.kt_end) {
+      ca.item += walk.slots;
+      setup_a(ca.item);
     }
   };
   auto advance_b = [&]() {
     if (cb.issued >= total_steps) return;
-    if (++cb.kt == k_steps) {
-      cb.kt = 0;
-      cb.tile += walk.slots;
-      setup_b(cb.tile);
+    if (++cb.kt == cb.kt_end) {
+      cb.item += walk.slots;
+      setup_b(cb.item);
     }
   };
 
@@ -326,18 +356,21 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_tiled_kernel(GemmP
       else fb[f - MT].lo = read_lo(rows_b, s, f - MT);
     }
   };
-  constexpr int NMFMA = MT * NT, NREAD = 2 * (MT + NT), NLOAD = A_GROUPS + B_GROUPS;
-  static_assert(NREAD <= NMFMA && 2 * A_GROUPS <= NMFMA && 2 * B_GROUPS <= NMFMA, "one read slot per MFMA, one load slot per two");
+  // Per half step: NMFMA MFMAs, NREAD LDS reads, A_GROUPS or B_GROUPS global->LDS loads, the
+  // memory instructions spread evenly behind the MFMAs (slot t gets reads [t*RPS, (t+1)*RPS)
+  // and load l when l*NMFMA/GROUPS == t).
+  constexpr int NMFMA = MT * NT, NREAD = 2 * (MT + NT);
+  constexpr int RPS = (NREAD + NMFMA - 1) / NMFMA;
+  static_assert(A_GROUPS <= NMFMA && B_GROUPS <= NMFMA, "at most one load slot per MFMA");
 
   // ---- prologue: A(0) B(0) A(1) B(1) in flight, first fragments in registers
-  setup_a(ca.tile);
-  setup_b(cb.tile);
+  setup_a(ca.item);
+  setup_b(cb.item);
   issue_a(); advance_a();
   issue_b(); advance_b();
   issue_a(); advance_a();
   issue_b(); advance_b();
-  if (KTAIL) wait_loads_and_barrier<0>();
-  else wait_loads_and_barrier<A_GROUPS + B_GROUPS>();
+  wait_loads_and_barrier<A_GROUPS + B_GROUPS>();
 #pragma unroll
   for (int u = 0; u < NREAD; ++u) read_one(xa, xb, lds + a_rd_base, lds + b_rd_base, 0, u);
 
@@ -407,12 +440,46 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_tiled_kernel(GemmP
     __builtin_amdgcn_sched_barrier(0);
   };
 
+  // ---- split-K: raw fp32 partial sums of this item to partial[split][m][n] (same lane layout
+  // as the epilogue: 4 consecutive n per lane, one 16-byte store when aligned)
+  auto store_partial = [&](int m0, int n0, int split) {
+    float* base = p.partial + (size_t)split * p.M * p.N;
+    const bool vec = (p.N & 3) == 0;
+#pragma unroll
+    for (int i = 0; i < MT; ++i) {
+      const int m = m0 + wm * WTM + i * 32 + l32;
+#pragma unroll
+      for (int j = 0; j < NT; ++j) {
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          const int n = n0 + wn * WTN + j * 32 + 8 * q + 4 * half;
+          const v4f v = {acc[i][j][4 * q], acc[i][j][4 * q + 1], acc[i][j][4 * q + 2], acc[i][j][4 * q + 3]};
+          if (m < p.M) {
+            float* dst = base + (size_t)m * p.N + n;
+            if (vec && n + 3 < p.N) {
+              *(v4f*)dst = v;
+            } else {
+#pragma unroll
+              for (int e = 0; e < 4; ++e)
+                if (n + e < p.N) dst[e] = v[e];
+            }
+          }
+        }
+#pragma unroll
+        for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.0f;
+      }
+    }
+    __builtin_amdgcn_sched_barrier(0);
+  };
+
   int sa = 0, sb = 0;  // stages holding the step being computed
   // Tile loop around the K loop (rather than one flat loop with a conditional epilogue):
   // the accumulators then have one simple live range per tile, which the register
   // allocator keeps in place.
-  for (int c_tile = walk.slot; c_tile < walk.chunk_len; c_tile += walk.slots) {
-    for (int kt = 0; kt < k_steps; ++kt) {
+  for (int c_item = walk.slot; c_item < walk.chunk_len; c_item += walk.slots) {
+    const int c_split = item_split(c_item);
+    for (int kt = split_begin(c_split); kt < split_end(c_split); ++kt) {
       const uint8_t* cur_a = lds + a_rd_base + sa * STAGE_A;
       const uint8_t* cur_b = lds + b_rd_base + sb * STAGE_B;
       sa = (sa + 1 == kStagesA) ? 0 : sa + 1;
@@ -426,70 +493,109 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_tiled_kernel(GemmP
       //     interleaving: every wave-level memory instruction hides behind an MFMA, and the
       //     load queue never holds more than the matrix pipe can cover.
       __builtin_amdgcn_sched_barrier(0);
-      if (!KTAIL) {
+      {
         const uint8_t* gb = l_b + (size_t)cb.kt * kStepK;
+        const bool real = !KTAIL || cb.kt < k_full || tail_chunk_ok;
         uint8_t* wb = lds + LDS_B0 + (cb.issued % kStagesB) * STAGE_B + wave * 1024;
         ++cb.issued;
 #pragma unroll
         for (int t = 0; t < NMFMA; ++t) {
           mfma_one(xa, xb, t);
-          if ((t & 1) == 0 && t / 2 < B_GROUPS) load_chunk_to_lds(gb + b_off[t / 2], wb + NW * (t / 2) * 1024);
-          if (t < NREAD) read_one(ya, yb, cur_a, cur_b, 1, t);
+#pragma unroll
+          for (int l = 0; l < B_GROUPS; ++l)
+            if (l * NMFMA / B_GROUPS == t) load_chunk_to_lds(chunk_src(gb, b_off[l], real), wb + NW * l * 1024);
+#pragma unroll
+          for (int u = t * RPS; u < (t + 1) * RPS; ++u)
+            if (u < NREAD) read_one(ya, yb, cur_a, cur_b, 1, u);
           __builtin_amdgcn_sched_barrier(0);
         }
-      } else {
-        issue_b();
-#pragma unroll
-        for (int t = 0; t < NMFMA; ++t) {
-          mfma_one(xa, xb, t);
-          if (t < NREAD) read_one(ya, yb, cur_a, cur_b, 1, t);
-        }
-        __builtin_amdgcn_sched_barrier(0);
       }
       advance_b();
 
       // own loads of A(g+1) and B(g+1) have landed (B(g+2) may still be in flight); past the
       // barrier everyone's have, and every wave is done reading this step's stages
-      if (KTAIL) wait_loads_and_barrier<0>();
-      else wait_loads_and_barrier<B_GROUPS>();
+      wait_loads_and_barrier<B_GROUPS>();
 
       // [B] MFMAs on y* (second K half); behind them the loads of A(g+2) into the A stage just
       //     released and the LDS reads of step g+1's first half (-> x*; at the end of a tile
       //     these already belong to the next tile)
       __builtin_amdgcn_sched_barrier(0);
-      if (!KTAIL) {
+      {
         const uint8_t* ga = l_a + (size_t)ca.kt * kStepK;
+        const bool real = !KTAIL || ca.kt < k_full || tail_chunk_ok;
         uint8_t* wa = lds + (ca.issued % kStagesA) * STAGE_A + wave * 1024;
         ++ca.issued;
 #pragma unroll
         for (int t = 0; t < NMFMA; ++t) {
           mfma_one(ya, yb, t);
-          if ((t & 1) == 0 && t / 2 < A_GROUPS) load_chunk_to_lds(ga + a_off[t / 2], wa + NW * (t / 2) * 1024);
-          if (t < NREAD) read_one(xa, xb, nxt_a, nxt_b, 0, t);
+#pragma unroll
+          for (int l = 0; l < A_GROUPS; ++l)
+            if (l * NMFMA / A_GROUPS == t) load_chunk_to_lds(chunk_src(ga, a_off[l], real), wa + NW * l * 1024);
+#pragma unroll
+          for (int u = t * RPS; u < (t + 1) * RPS; ++u)
+            if (u < NREAD) read_one(xa, xb, nxt_a, nxt_b, 0, u);
           __builtin_amdgcn_sched_barrier(0);
         }
-      } else {
-        issue_a();
-#pragma unroll
-        for (int t = 0; t < NMFMA; ++t) {
-          mfma_one(ya, yb, t);
-          if (t < NREAD) read_one(xa, xb, nxt_a, nxt_b, 0, t);
-        }
-        __builtin_amdgcn_sched_barrier(0);
       }
       advance_a();
     }
     {
       int tm, tn;
-      tile_coords(walk.chunk_begin + c_tile, p.tiles_m, p.tiles_n, p.group_m, tm, tn);
+      tile_coords(item_tile(c_item), p.tiles_m, p.tiles_n, p.group_m, tm, tn);
       const int m0 = tm * BM, n0 = tn * BN;
-      const bool interior = (m0 + BM <= p.M) && (n0 + BN <= p.N) && ((p.ldc & 3) == 0) &&
-                            ((reinterpret_cast<uintptr_t>(p.c) & 7) == 0);
-      if (interior) epilogue(m0, n0, std::true_type{});
-      else epilogue(m0, n0, std::false_type{});
+      if (EPI == kEpiPartial) {
+        store_partial(m0, n0, c_split);
+      } else {
+        const bool interior = (m0 + BM <= p.M) && (n0 + BN <= p.N) && ((p.ldc & 3) == 0) &&
+                              ((reinterpret_cast<uintptr_t>(p.c) & 7) == 0);
+        if (interior) epilogue(m0, n0, std::true_type{});
+        else epilogue(m0, n0, std::false_type{});
+      }
     }
   }
   __builtin_amdgcn_s_waitcnt(0x0070);  // the trailing dummy loads must land before LDS is released
+}
+
+// Second pass of a split-K launch: sums the splits' partials in a fixed order (results do not
+// depend on scheduling), applies the scales and the bias and rounds to bf16. One thread per
+// 4 consecutive columns.
+__global__ __launch_bounds__(256) void splitk_finalize_kernel(GemmParams p) {
+  const long quads_per_row = (p.N + 3) / 4;
+  const long idx = (long)blockIdx.x * 256 + threadIdx.x;
+  if (idx >= quads_per_row * p.M) return;
+  const int m = (int)(idx / quads_per_row);
+  const int n = (int)(idx % quads_per_row) * 4;
+  const size_t plane = (size_t)p.M * p.N;
+  const float* src = p.partial + (size_t)m * p.N + n;
+  const bool vec = (p.N & 3) == 0;  // then n + 3 < N and every row start is 16-byte aligned
+  v4f sum = {0.f, 0.f, 0.f, 0.f};
+  for (int s = 0; s < p.splits; ++s) {
+    if (vec) {
+      sum += *(const v4f*)(src + s * plane);
+    } else {
+#pragma unroll
+      for (int e = 0; e < 4; ++e)
+        if (n + e < p.N) sum[e] += src[s * plane + e];
+    }
+  }
+  const float sa_m = p.a_scale[m];
+  float r[4];
+#pragma unroll
+  for (int e = 0; e < 4; ++e) {
+    const int ne = min(n + e, p.N - 1);
+    const float t = sum[e] * sa_m;
+    r[e] = p.bias ? __builtin_fmaf(t, p.b_scale[ne], bf16_to_f32(p.bias[ne])) : t * p.b_scale[ne];
+  }
+  const uint32_t lo = pack_bf16x2(r[0], r[1]), hi = pack_bf16x2(r[2], r[3]);
+  uint16_t* dst = p.c + (size_t)m * p.ldc + n;
+  if (n + 3 < p.N && ((p.ldc & 3) == 0) && ((reinterpret_cast<uintptr_t>(p.c) & 7) == 0)) {
+    *(v2u*)dst = (v2u){lo, hi};
+  } else {
+    dst[0] = (uint16_t)lo;
+    if (n + 1 < p.N) dst[1] = (uint16_t)(lo >> 16);
+    if (n + 2 < p.N) dst[2] = (uint16_t)hi;
+    if (n + 3 < p.N) dst[3] = (uint16_t)(hi >> 16);
+  }
 }
 
 // ------------------------------------------------------------------------------------
@@ -760,16 +866,96 @@ int check_shape(int64_t M, int64_t N, int64_t K) {
   return MI355X_FP8_OK;
 }
 
-template <int BM, int BN, int WAVES_M, int WAVES_N, bool KTAIL, bool HAS_BIAS>
+// ---- tiled-kernel plans: tile configuration x split-K factor
+struct TileConfig {
+  int bm, bn, wgs_per_cu;
+  float us_per_step;        // one 128-byte K step of a work item, every workgroup slot busy
+  float us_per_step_alone;  // the same with at most one workgroup per CU
+  float us_per_item;        // pipeline refill + epilogue of one work item
+  float stream_bytes_per_us;  // operand bytes per microsecond the configuration can stream from HBM
+};
+constexpr int kNumTileConfigs = 2;
+// Measured on MI355X with normally distributed operands (clock under sustained MFMA load).
+constexpr TileConfig kTileConfigs[kNumTileConfigs] = {
+    {256, 256, tiled_wgs_per_cu(256, 256), 1.30f, 1.30f, 6.0f, 3.6e6f},
+    {128, 128, tiled_wgs_per_cu(128, 128), 1.00f, 0.62f, 5.0f, 4.4e6f},
+};
+constexpr int kMaxSplits = 16;
+
+struct TiledPlan {
+  int config, splits, steps_per_split;
+};
+
+inline int k_steps_of(int64_t K) { return (int)((K + kStepK - 1) / kStepK); }
+
+// Splits actually used when `want` are asked for: every split gets the same whole number of
+// steps and none is empty.
+inline void normalise_splits(int k_steps, int want, int& splits, int& sps) {
+  want = want < 1 ? 1 : (want > k_steps ? k_steps : want);
+  sps = (k_steps + want - 1) / want;
+  splits = (k_steps + sps - 1) / sps;
+}
+
+// Estimated run time of a plan. Work items are dealt to 256 * wgs_per_cu workgroup slots in
+// rounds; a last round that fills at most one slot per CU runs at the faster stand-alone
+// rate. The operands cannot arrive faster than the configuration streams from HBM. Split
+// plans add a launch and the partial sums' trip through memory (written once, read once).
+inline float plan_cost_us(int64_t M, int64_t N, int64_t K, int config, int splits, int sps) {
+  const TileConfig& c = kTileConfigs[config];
+  const long tiles = ((M + c.bm - 1) / c.bm) * ((N + c.bn - 1) / c.bn);
+  const long items = tiles * splits;
+  const long slots = (long)kNumCu * c.wgs_per_cu;
+  const long full_rounds = items / slots, rest = items % slots;
+  float t = full_rounds * (sps * c.us_per_step + c.us_per_item);
+  if (rest) t += sps * (rest <= kNumCu ? c.us_per_step_alone : c.us_per_step) + c.us_per_item;
+  const float stream = ((float)M * (float)K + (float)N * (float)K) / c.stream_bytes_per_us;
+  if (t < stream) t = stream;
+  if (splits > 1) t += 4.0f + 2.0f * (float)splits * (float)M * (float)N * 4.0f / 3.5e6f;
+  return t;
+}
+
+// Cheapest plan by the model above; `max_splits` = 1 restricts it to plans without workspace.
+inline TiledPlan plan_tiled(int64_t M, int64_t N, int64_t K, int force_config, int force_splits,
+                            int max_splits) {
+  const int k_steps = k_steps_of(K);
+  TiledPlan best = {0, 1, k_steps};
+  float best_cost = -1.0f;
+  for (int c = 0; c < kNumTileConfigs; ++c) {
+    if (force_config >= 0 && c != force_config) continue;
+    for (int want = 1; want <= max_splits; ++want) {
+      if (force_splits > 0 && want != force_splits) continue;
+      int splits, sps;
+      normalise_splits(k_steps, want, splits, sps);
+      if (force_splits <= 0 && splits != want) continue;  // duplicate of a smaller request
+      const float cost = plan_cost_us(M, N, K, c, splits, sps);
+      if (best_cost < 0.0f || cost < best_cost) {
+        best_cost = cost;
+        best = {c, splits, sps};
+      }
+    }
+  }
+  return best;
+}
+
+// variant word: bits 0..7 kernel family, bits 8..15 tile configuration + 1 (0 = automatic),
+// bits 16..23 split-K factor (0 = automatic)
+inline TiledPlan plan_from_variant(int64_t M, int64_t N, int64_t K, int variant, int max_splits) {
+  const int cfg = ((variant >> 8) & 0xff) - 1;
+  const int spl = (variant >> 16) & 0xff;
+  return plan_tiled(M, N, K, cfg, spl, spl > 0 ? spl : max_splits);
+}
+
+template <int BM, int BN, int WAVES_M, int WAVES_N, bool KTAIL, int EPI>
 int launch_tiled(GemmParams p, hipStream_t stream) {
   constexpr int threads = WAVES_M * WAVES_N * 64;
-  constexpr size_t lds_bytes = (size_t)(kStagesA * BM + kStagesB * BN) * kStepK;
+  constexpr size_t lds_bytes = tiled_lds_bytes(BM, BN);
   p.tiles_m = (p.M + BM - 1) / BM;
   p.tiles_n = (p.N + BN - 1) / BN;
   p.group_m = 4;
-  const long total = (long)p.tiles_m * p.tiles_n;
-  long grid = total < kNumCu ? ((total + kNumXcd - 1) / kNumXcd) * kNumXcd : kNumCu;
-  auto kern = gemm_tiled_kernel<BM, BN, WAVES_M, WAVES_N, KTAIL, HAS_BIAS>;
+  const long total = (long)p.tiles_m * p.tiles_n * p.splits;
+  const long slots = (long)kNumCu * tiled_wgs_per_cu(BM, BN);
+  long grid = total < slots ? ((total + kNumXcd - 1) / kNumXcd) * kNumXcd : slots;
+  auto kern = gemm_tiled_kernel<BM, BN, WAVES_M, WAVES_N, KTAIL, EPI>;
   static bool attr_set = false;  // raising the dynamic LDS limit is idempotent; races are harmless
   if (!attr_set) {
     hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize,
@@ -780,7 +966,26 @@ int launch_tiled(GemmParams p, hipStream_t stream) {
   hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(threads), lds_bytes, stream, p);
   hipError_t e = hipGetLastError();
   if (e != hipSuccess) return fail(MI355X_FP8_ELAUNCH, "tiled kernel launch: %s", hipGetErrorString(e));
+  if (EPI == kEpiPartial) {
+    const long quads = (long)p.M * ((p.N + 3) / 4);
+    hipLaunchKernelGGL(splitk_finalize_kernel, dim3((unsigned)((quads + 255) / 256)), dim3(256), 0, stream, p);
+    e = hipGetLastError();
+    if (e != hipSuccess) return fail(MI355X_FP8_ELAUNCH, "split-K finalize launch: %s", hipGetErrorString(e));
+  }
   return MI355X_FP8_OK;
+}
+
+template <int BM, int BN, int WAVES_M, int WAVES_N>
+int launch_tiled_config(const GemmParams& p, hipStream_t s) {
+  const bool ktail = p.K % kStepK;
+  if (p.splits > 1)
+    return ktail ? launch_tiled<BM, BN, WAVES_M, WAVES_N, true, kEpiPartial>(p, s)
+                 : launch_tiled<BM, BN, WAVES_M, WAVES_N, false, kEpiPartial>(p, s);
+  if (p.bias)
+    return ktail ? launch_tiled<BM, BN, WAVES_M, WAVES_N, true, kEpiBias>(p, s)
+                 : launch_tiled<BM, BN, WAVES_M, WAVES_N, false, kEpiBias>(p, s);
+  return ktail ? launch_tiled<BM, BN, WAVES_M, WAVES_N, true, kEpiPlain>(p, s)
+               : launch_tiled<BM, BN, WAVES_M, WAVES_N, false, kEpiPlain>(p, s);
 }
 
 template <int MT, int NTW, int DEPTH, int KW>
@@ -816,15 +1021,18 @@ int mi355x_fp8_rowwise_select_variant(int64_t M, int64_t N, int64_t K) {
 }
 
 size_t mi355x_fp8_rowwise_workspace_bytes(int64_t M, int64_t N, int64_t K, int variant) {
-  (void)M; (void)N; (void)K; (void)variant;
-  return 0;  // both kernel families reduce on chip
+  if (check_shape(M, N, K) != MI355X_FP8_OK) return 0;
+  if ((variant & 0xff) == MI355X_FP8_VARIANT_AUTO)
+    variant = (variant & ~0xff) | mi355x_fp8_rowwise_select_variant(M, N, K);
+  if ((variant & 0xff) != MI355X_FP8_VARIANT_TILED) return 0;  // the skinny kernel reduces on chip
+  const TiledPlan plan = plan_from_variant(M, N, K, variant, kMaxSplits);
+  return plan.splits > 1 ? (size_t)plan.splits * (size_t)M * (size_t)N * sizeof(float) : 0;
 }
 
 int mi355x_fp8_rowwise_gemm(const void* a, const void* b, const float* a_scale, const float* b_scale,
                             const void* bias, void* c, int64_t M, int64_t N, int64_t K, int64_t lda,
                             int64_t ldb, int64_t ldc, void* workspace, size_t workspace_bytes,
                             int variant, void* stream) {
-  (void)workspace; (void)workspace_bytes;
   int st = check_shape(M, N, K);
   if (st != MI355X_FP8_OK) return st;
   if (!a || !b || !a_scale || !b_scale || !c) return fail(MI355X_FP8_EINVAL, "null operand pointer");
@@ -837,6 +1045,10 @@ int mi355x_fp8_rowwise_gemm(const void* a, const void* b, const float* a_scale, 
     return fail(MI355X_FP8_EINVAL, "misaligned scale, bias or output pointer");
   if (lda * 256 > (int64_t)UINT32_MAX || ldb * 256 > (int64_t)UINT32_MAX)
     return fail(MI355X_FP8_ENOTSUP, "leading dimension too large");
+  if (variant < 0 || (variant >> 24) || ((variant >> 8) & 0xff) > kNumTileConfigs)
+    return fail(MI355X_FP8_EINVAL, "unknown variant 0x%x", variant);
+  const int plan_bits = variant & ~0xff;
+  variant &= 0xff;
   if (variant == MI355X_FP8_VARIANT_AUTO) variant = mi355x_fp8_rowwise_select_variant(M, N, K);
   if (variant == MI355X_FP8_VARIANT_SKINNY && M > kSkinnyMaxM)
     return fail(MI355X_FP8_ENOTSUP, "skinny variant handles M <= %d (got %lld)", kSkinnyMaxM, (long long)M);
@@ -848,6 +1060,7 @@ int mi355x_fp8_rowwise_gemm(const void* a, const void* b, const float* a_scale, 
   p.M = (int)M; p.N = (int)N; p.K = (int)K;
   p.lda = lda; p.ldb = ldb; p.ldc = ldc;
   p.tiles_m = p.tiles_n = 0; p.group_m = 1;
+  p.splits = 1; p.steps_per_split = k_steps_of(K); p.partial = nullptr;
   hipStream_t s = (hipStream_t)stream;
 
   switch (variant) {
@@ -855,8 +1068,28 @@ int mi355x_fp8_rowwise_gemm(const void* a, const void* b, const float* a_scale, 
       // b_scale is read 16 bytes at a time on full tiles
       if (reinterpret_cast<uintptr_t>(b_scale) & 15 || (bias && (reinterpret_cast<uintptr_t>(bias) & 7)))
         return fail(MI355X_FP8_ENOTSUP, "tiled variant needs b_scale 16-byte and bias 8-byte aligned");
-      if (K % kStepK) return bias ? launch_tiled<256, 256, 2, 2, true, true>(p, s) : launch_tiled<256, 256, 2, 2, true, false>(p, s);
-      return bias ? launch_tiled<256, 256, 2, 2, false, true>(p, s) : launch_tiled<256, 256, 2, 2, false, false>(p, s);
+      {
+        // A caller that brought no (or too little) workspace gets the best plan that needs none,
+        // unless it asked for a split factor by name.
+        TiledPlan plan = plan_from_variant(M, N, K, plan_bits, kMaxSplits);
+        const size_t need = plan.splits > 1 ? (size_t)plan.splits * M * N * sizeof(float) : 0;
+        if (need && (!workspace || workspace_bytes < need)) {
+          if ((plan_bits >> 16) & 0xff)
+            return fail(MI355X_FP8_EINVAL, "split-K factor %d needs %zu bytes of workspace (got %zu)",
+                        plan.splits, need, workspace ? workspace_bytes : (size_t)0);
+          plan = plan_from_variant(M, N, K, plan_bits, 1);
+        }
+        if (plan.splits > 1 && (reinterpret_cast<uintptr_t>(workspace) & 15))
+          return fail(MI355X_FP8_EINVAL, "workspace must be 16-byte aligned");
+        p.splits = plan.splits;
+        p.steps_per_split = plan.steps_per_split;
+        p.partial = plan.splits > 1 ? (float*)workspace : nullptr;
+        switch (plan.config) {
+          case 0: return launch_tiled_config<256, 256, 2, 2>(p, s);
+          case 1: return launch_tiled_config<128, 128, 2, 2>(p, s);
+          default: return fail(MI355X_FP8_EINVAL, "unknown tile configuration %d", plan.config);
+        }
+      }
     case MI355X_FP8_VARIANT_SKINNY:
       // 16-row blocks of A | B tiles per wave | steps in flight per wave (sized to 128 VGPRs)
 #ifndef SKCFG
