@@ -332,18 +332,14 @@ void gemm_tiled_kernel(GemmParams p) {
     return (v8i){f.lo[0], f.lo[1], f.lo[2], f.lo[3], f.hi[0], f.hi[1], f.hi[2], f.hi[3]};
   };
 
-  v16f acc[MT][NT];
-#pragma unroll
-  for (int i = 0; i < MT; ++i)
-#pragma unroll
-    for (int j = 0; j < NT; ++j)
-#pragma unroll
-      for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.0f;
+  v16f acc[MT][NT];  // defined by the first step of every work item
 
   // t-th MFMA of a half step (t = i*NT + j) on fragment set (fa, fb)
-  auto mfma_one = [&](const Frag (&fa)[MT], const Frag (&fb)[NT], int t) {
+  // (fresh: the block's first MFMA of a tile starts from zero instead of the old contents)
+  auto mfma_one = [&](const Frag (&fa)[MT], const Frag (&fb)[NT], int t, bool fresh) {
     const int i = t / NT, j = t % NT;
-    acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(as_v8(fb[j]), as_v8(fa[i]), acc[i][j], 0, 0, 0, 0, 0, 0);
+    const v16f zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+    acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(as_v8(fb[j]), as_v8(fa[i]), fresh ? zero : acc[i][j], 0, 0, 0, 0, 0, 0);
   };
   // u-th of the 2*(MT+NT) LDS reads that fill fragment set (fa, fb) with K half s
   auto read_one = [&](Frag (&fa)[MT], Frag (&fb)[NT], const uint8_t* rows_a, const uint8_t* rows_b, int s, int u) {
@@ -374,67 +370,117 @@ void gemm_tiled_kernel(GemmParams p) {
 #pragma unroll
   for (int u = 0; u < NREAD; ++u) read_one(xa, xb, lds + a_rd_base, lds + b_rd_base, 0, u);
 
-  // ---- epilogue. For every (i, j) sub-tile the lane holds row m = .. + l32 and the columns
-  // n = .. + 8*q + 4*half + e (register v = 4*q + e). All scale and bias values the lane
-  // needs are fetched up front (one memory latency per tile), then each sub-tile is scaled,
-  // rounded to bf16 by the hardware pack-convert and stored; INTERIOR tiles use 8-byte
-  // stores, edge tiles guard every element. Accumulators are cleared on the way out.
-  auto epilogue = [&](int m0, int n0, auto interior_tag) {
-    constexpr bool INTERIOR = decltype(interior_tag)::value;
-    float sam[MT], sbn[NT][4][4], bn[NT][4][4];
+  // ---- epilogue. The MFMA leaves lane (l32, half) with row l32 of every 32x32 block and the
+  // columns 8*q + 4*half + e (register 4*q + e): storing from there would touch 32 rows per
+  // instruction. Instead each 32-row block of the wave's tile is turned through LDS, PASS_J
+  // 32-column blocks at a time, as fp32 already multiplied by a_scale[m]; read back, a lane
+  // holds 8 consecutive columns of one row, multiplies by b_scale (adds the bias), rounds to
+  // bf16 once and stores 16 bytes, so a wave-wide store covers whole rows of the pass.
+  // A lane's 8 columns are the same for every row, which keeps its b_scale / bias working
+  // set at 8 values per pass column group.
+  //
+  // The turn-table is the wave's own share (the 1 KB groups it fills itself) of the B stage
+  // that held this tile's last step: every wave finished reading that stage before the
+  // step's barrier, and only this wave will load into these groups again. A pass row is CPR
+  // 16-byte chunks; chunk c of row r sits at chunk position c ^ key(r).
+  constexpr int PASS_J = B_GROUPS / 4;          // 32-column blocks per pass (4 KB of fp32 each)
+  constexpr int NJP = NT / PASS_J;              // passes per 32-row block
+  constexpr int CPR = PASS_J * 8;               // 16-byte chunks per pass row
+  constexpr int ROW_BYTES = CPR * 16;
+  constexpr int ROWS_PER_GROUP = 1024 / ROW_BYTES;
+  constexpr int LPR = CPR / 2;                  // lanes per row when reading back (2 chunks each)
+  constexpr int ROWS_PER_READ = 64 / LPR;
+  static_assert(B_GROUPS % 4 == 0 && NT % PASS_J == 0 && (CPR == 8 || CPR == 16), "turn-table geometry");
+  auto epilogue = [&](int m0, int n0, auto aligned_tag, uint8_t* free_b_stage) {
+    constexpr bool ALIGNED = decltype(aligned_tag)::value;  // whole tile inside C, rows 16-byte aligned
+    auto row_addr = [&](int r) -> uint8_t* {
+      return free_b_stage + (wave + NW * (r / ROWS_PER_GROUP)) * 1024 + (r % ROWS_PER_GROUP) * ROW_BYTES;
+    };
+    auto key = [](int r) { return (r * CPR / 16) % CPR; };
+    // The lane-dependent addresses below are the same for every tile; derived from an opaque
+    // copy of the lane id they are recomputed here (a few integer operations) instead of
+    // being hoisted out of the tile loop, where they would occupy registers through the K loop.
+    int lane_e = lane;
+    asm volatile("" : "+v"(lane_e));
+    const int l32 = lane_e & 31, half = lane_e >> 5;
+    uint8_t* const wr_row = row_addr(l32);
+    const int wr_key = key(l32);
+    const int rd_row = lane_e / LPR, rd_col = (lane_e % LPR) * 8;  // column of the pass row this lane stores
+
+    float sam[MT], sbv[NJP][8], bv[NJP][8];
 #pragma unroll
     for (int i = 0; i < MT; ++i) sam[i] = p.a_scale[min(m0 + wm * WTM + i * 32 + l32, p.M - 1)];
 #pragma unroll
-    for (int j = 0; j < NT; ++j)
+    for (int jp = 0; jp < NJP; ++jp) {
+      const int n = n0 + wn * WTN + jp * PASS_J * 32 + rd_col;
+      if (ALIGNED) {
+        const v4f s0 = *(const v4f*)(p.b_scale + n), s1 = *(const v4f*)(p.b_scale + n + 4);
 #pragma unroll
-      for (int q = 0; q < 4; ++q) {
-        const int n = n0 + wn * WTN + j * 32 + 8 * q + 4 * half;
-        if (INTERIOR) {
-          const v4f s4 = *(const v4f*)(p.b_scale + n);
+        for (int e = 0; e < 4; ++e) sbv[jp][e] = s0[e], sbv[jp][4 + e] = s1[e];
+        if (HAS_BIAS) {
+          const us4 b0 = *(const us4*)(p.bias + n), b1 = *(const us4*)(p.bias + n + 4);
 #pragma unroll
-          for (int e = 0; e < 4; ++e) sbn[j][q][e] = s4[e];
-          if (HAS_BIAS) {
-            const us4 b4 = *(const us4*)(p.bias + n);
+          for (int e = 0; e < 4; ++e) bv[jp][e] = bf16_to_f32(b0[e]), bv[jp][4 + e] = bf16_to_f32(b1[e]);
+        }
+      } else {
 #pragma unroll
-            for (int e = 0; e < 4; ++e) bn[j][q][e] = bf16_to_f32(b4[e]);
-          }
-        } else {
-#pragma unroll
-          for (int e = 0; e < 4; ++e) {
-            sbn[j][q][e] = p.b_scale[min(n + e, p.N - 1)];
-            if (HAS_BIAS) bn[j][q][e] = bf16_to_f32(p.bias[min(n + e, p.N - 1)]);
-          }
+        for (int e = 0; e < 8; ++e) {
+          sbv[jp][e] = p.b_scale[min(n + e, p.N - 1)];
+          if (HAS_BIAS) bv[jp][e] = bf16_to_f32(p.bias[min(n + e, p.N - 1)]);
         }
       }
+    }
 #pragma unroll
     for (int i = 0; i < MT; ++i) {
-      const int m = m0 + wm * WTM + i * 32 + l32;
-      uint16_t* crow = p.c + (size_t)m * p.ldc + n0 + wn * WTN + 4 * half;
 #pragma unroll
-      for (int j = 0; j < NT; ++j) {
+      for (int jp = 0; jp < NJP; ++jp) {
         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-        for (int q = 0; q < 4; ++q) {
-          float r[4];
+        for (int jj = 0; jj < PASS_J; ++jj) {
+          const int j = jp * PASS_J + jj;
 #pragma unroll
-          for (int e = 0; e < 4; ++e) {
-            const float t = acc[i][j][4 * q + e] * sam[i];
-            r[e] = HAS_BIAS ? __builtin_fmaf(t, sbn[j][q][e], bn[j][q][e]) : t * sbn[j][q][e];
+          for (int q = 0; q < 4; ++q) {
+            v4f t;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) t[e] = acc[i][j][4 * q + e] * sam[i];
+            *(v4f*)(wr_row + (((jj * 8 + 2 * q + half) ^ wr_key) * 16)) = t;
           }
-          const uint32_t lo = pack_bf16x2(r[0], r[1]), hi = pack_bf16x2(r[2], r[3]);
-          uint16_t* dst = crow + j * 32 + 8 * q;
-          if (INTERIOR) {
-            *(v2u*)dst = (v2u){lo, hi};
-          } else if (m < p.M) {
-            const int n = n0 + wn * WTN + j * 32 + 8 * q + 4 * half;
-            if (n + 0 < p.N) dst[0] = (uint16_t)lo;
-            if (n + 1 < p.N) dst[1] = (uint16_t)(lo >> 16);
-            if (n + 2 < p.N) dst[2] = (uint16_t)hi;
-            if (n + 3 < p.N) dst[3] = (uint16_t)(hi >> 16);
-          }
+          __builtin_amdgcn_sched_barrier(0);  // keeps the live set small: one block at a time
         }
+        const int n = n0 + wn * WTN + jp * PASS_J * 32 + rd_col;
+        constexpr int ITERS = 32 / ROWS_PER_READ;
+        v4f lo4[ITERS], hi4[ITERS];
 #pragma unroll
-        for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.0f;
+        for (int it = 0; it < ITERS; ++it) {
+          const int r = it * ROWS_PER_READ + rd_row;
+          const uint8_t* src = row_addr(r);
+          const int c0 = (rd_col / 4) ^ key(r);  // the lane's two chunks differ in bit 0 only
+          lo4[it] = *(const v4f*)(src + c0 * 16);
+          hi4[it] = *(const v4f*)(src + (c0 ^ 1) * 16);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int it = 0; it < ITERS; ++it) {
+          const int r = it * ROWS_PER_READ + rd_row;
+          float x[8];
+#pragma unroll
+          for (int e = 0; e < 4; ++e) x[e] = lo4[it][e], x[4 + e] = hi4[it][e];
+#pragma unroll
+          for (int e = 0; e < 8; ++e)
+            x[e] = HAS_BIAS ? __builtin_fmaf(x[e], sbv[jp][e], bv[jp][e]) : x[e] * sbv[jp][e];
+          const v4i out = {(int)pack_bf16x2(x[0], x[1]), (int)pack_bf16x2(x[2], x[3]),
+                           (int)pack_bf16x2(x[4], x[5]), (int)pack_bf16x2(x[6], x[7])};
+          const int m = m0 + wm * WTM + i * 32 + r;
+          uint16_t* dst = p.c + (size_t)m * p.ldc + n;
+          if (ALIGNED) {
+            *(v4i*)dst = out;
+          } else if (m < p.M) {
+#pragma unroll
+            for (int e = 0; e < 8; ++e)
+              if (n + e < p.N) dst[e] = (uint16_t)((unsigned)out[e / 2] >> (16 * (e & 1)));
+          }
+          __builtin_amdgcn_sched_barrier(0);
+        }
       }
     }
     __builtin_amdgcn_sched_barrier(0);
@@ -466,78 +512,96 @@ void gemm_tiled_kernel(GemmParams p) {
             }
           }
         }
-#pragma unroll
-        for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.0f;
       }
     }
     __builtin_amdgcn_sched_barrier(0);
   };
 
   int sa = 0, sb = 0;  // stages holding the step being computed
-  // Tile loop around the K loop (rather than one flat loop with a conditional epilogue):
-  // the accumulators then have one simple live range per tile, which the register
-  // allocator keeps in place.
+  // One K step. READ_NEXT: fetch the first-half fragments of the following step behind the
+  // second-half MFMAs (left out on a tile's last step, so that the epilogue has those
+  // registers; the fragments are then read after it).
+  auto step = [&](auto first_tag, auto read_next_tag) {
+    constexpr bool FIRST = decltype(first_tag)::value;
+    constexpr bool READ_NEXT = decltype(read_next_tag)::value;
+    const uint8_t* cur_a = lds + a_rd_base + sa * STAGE_A;
+    const uint8_t* cur_b = lds + b_rd_base + sb * STAGE_B;
+    sa = (sa + 1 == kStagesA) ? 0 : sa + 1;
+    sb = (sb + 1 == kStagesB) ? 0 : sb + 1;
+    const uint8_t* nxt_a = lds + a_rd_base + sa * STAGE_A;
+    const uint8_t* nxt_b = lds + b_rd_base + sb * STAGE_B;
+
+    // [A] MFMAs on x* (first K half of this step). Behind them, one per MFMA: the LDS reads
+    //     of the second half (-> y*), and behind every other one a global->LDS load of
+    //     B(g+2) into the B stage released at the previous barrier. The fences pin this
+    //     interleaving: every wave-level memory instruction hides behind an MFMA, and the
+    //     load queue never holds more than the matrix pipe can cover.
+    __builtin_amdgcn_sched_barrier(0);
+    {
+      const uint8_t* gb = l_b + (size_t)cb.kt * kStepK;
+      const bool real = !KTAIL || cb.kt < k_full || tail_chunk_ok;
+      uint8_t* wb = lds + LDS_B0 + (cb.issued % kStagesB) * STAGE_B + wave * 1024;
+      ++cb.issued;
+#pragma unroll
+      for (int t = 0; t < NMFMA; ++t) {
+        mfma_one(xa, xb, t, FIRST);
+#pragma unroll
+        for (int l = 0; l < B_GROUPS; ++l)
+          if (l * NMFMA / B_GROUPS == t) load_chunk_to_lds(chunk_src(gb, b_off[l], real), wb + NW * l * 1024);
+#pragma unroll
+        for (int u = t * RPS; u < (t + 1) * RPS; ++u)
+          if (u < NREAD) read_one(ya, yb, cur_a, cur_b, 1, u);
+        __builtin_amdgcn_sched_barrier(0);
+      }
+    }
+    advance_b();
+
+    // own loads of A(g+1) and B(g+1) have landed (B(g+2) may still be in flight); past the
+    // barrier everyone's have, and every wave is done reading this step's stages
+    wait_loads_and_barrier<B_GROUPS>();
+
+    // [B] MFMAs on y* (second K half); behind them the loads of A(g+2) into the A stage just
+    //     released and the LDS reads of step g+1's first half (-> x*; at the end of a tile
+    //     these already belong to the next tile)
+    __builtin_amdgcn_sched_barrier(0);
+    {
+      const uint8_t* ga = l_a + (size_t)ca.kt * kStepK;
+      const bool real = !KTAIL || ca.kt < k_full || tail_chunk_ok;
+      uint8_t* wa = lds + (ca.issued % kStagesA) * STAGE_A + wave * 1024;
+      ++ca.issued;
+#pragma unroll
+      for (int t = 0; t < NMFMA; ++t) {
+        mfma_one(ya, yb, t, false);
+#pragma unroll
+        for (int l = 0; l < A_GROUPS; ++l)
+          if (l * NMFMA / A_GROUPS == t) load_chunk_to_lds(chunk_src(ga, a_off[l], real), wa + NW * l * 1024);
+#pragma unroll
+        for (int u = t * RPS; u < (t + 1) * RPS; ++u)
+          if (READ_NEXT && u < NREAD) read_one(xa, xb, nxt_a, nxt_b, 0, u);
+        __builtin_amdgcn_sched_barrier(0);
+      }
+    }
+    advance_a();
+  };
+  auto read_first_half = [&]() {
+#pragma unroll
+    for (int u = 0; u < NREAD; ++u)
+      read_one(xa, xb, lds + a_rd_base + sa * STAGE_A, lds + b_rd_base + sb * STAGE_B, 0, u);
+  };
+
+  // Item loop around the K loop. The first step of an item is its own copy of the step code
+  // whose first-half MFMAs start from zero: the accumulators then have one live range per
+  // item (defined there, dead after the epilogue) and need no clearing or copying between
+  // items.
   for (int c_item = walk.slot; c_item < walk.chunk_len; c_item += walk.slots) {
     const int c_split = item_split(c_item);
-    for (int kt = split_begin(c_split); kt < split_end(c_split); ++kt) {
-      const uint8_t* cur_a = lds + a_rd_base + sa * STAGE_A;
-      const uint8_t* cur_b = lds + b_rd_base + sb * STAGE_B;
-      sa = (sa + 1 == kStagesA) ? 0 : sa + 1;
-      sb = (sb + 1 == kStagesB) ? 0 : sb + 1;
-      const uint8_t* nxt_a = lds + a_rd_base + sa * STAGE_A;
-      const uint8_t* nxt_b = lds + b_rd_base + sb * STAGE_B;
-
-      // [A] MFMAs on x* (first K half of this step). Behind them, one per MFMA: the LDS reads
-      //     of the second half (-> y*), and behind every other one a global->LDS load of
-      //     B(g+2) into the B stage released at the previous barrier. The fences pin this
-      //     interleaving: every wave-level memory instruction hides behind an MFMA, and the
-      //     load queue never holds more than the matrix pipe can cover.
-      __builtin_amdgcn_sched_barrier(0);
-      {
-        const uint8_t* gb = l_b + (size_t)cb.kt * kStepK;
-        const bool real = !KTAIL || cb.kt < k_full || tail_chunk_ok;
-        uint8_t* wb = lds + LDS_B0 + (cb.issued % kStagesB) * STAGE_B + wave * 1024;
-        ++cb.issued;
-#pragma unroll
-        for (int t = 0; t < NMFMA; ++t) {
-          mfma_one(xa, xb, t);
-#pragma unroll
-          for (int l = 0; l < B_GROUPS; ++l)
-            if (l * NMFMA / B_GROUPS == t) load_chunk_to_lds(chunk_src(gb, b_off[l], real), wb + NW * l * 1024);
-#pragma unroll
-          for (int u = t * RPS; u < (t + 1) * RPS; ++u)
-            if (u < NREAD) read_one(ya, yb, cur_a, cur_b, 1, u);
-          __builtin_amdgcn_sched_barrier(0);
-        }
-      }
-      advance_b();
-
-      // own loads of A(g+1) and B(g+1) have landed (B(g+2) may still be in flight); past the
-      // barrier everyone's have, and every wave is done reading this step's stages
-      wait_loads_and_barrier<B_GROUPS>();
-
-      // [B] MFMAs on y* (second K half); behind them the loads of A(g+2) into the A stage just
-      //     released and the LDS reads of step g+1's first half (-> x*; at the end of a tile
-      //     these already belong to the next tile)
-      __builtin_amdgcn_sched_barrier(0);
-      {
-        const uint8_t* ga = l_a + (size_t)ca.kt * kStepK;
-        const bool real = !KTAIL || ca.kt < k_full || tail_chunk_ok;
-        uint8_t* wa = lds + (ca.issued % kStagesA) * STAGE_A + wave * 1024;
-        ++ca.issued;
-#pragma unroll
-        for (int t = 0; t < NMFMA; ++t) {
-          mfma_one(ya, yb, t);
-#pragma unroll
-          for (int l = 0; l < A_GROUPS; ++l)
-            if (l * NMFMA / A_GROUPS == t) load_chunk_to_lds(chunk_src(ga, a_off[l], real), wa + NW * l * 1024);
-#pragma unroll
-          for (int u = t * RPS; u < (t + 1) * RPS; ++u)
-            if (u < NREAD) read_one(xa, xb, nxt_a, nxt_b, 0, u);
-          __builtin_amdgcn_sched_barrier(0);
-        }
-      }
-      advance_a();
+    const int n_steps = split_end(c_split) - split_begin(c_split);
+    if (n_steps == 1) {
+      step(std::true_type{}, std::false_type{});
+    } else {
+      step(std::true_type{}, std::true_type{});
+      for (int k = 2; k < n_steps; ++k) step(std::false_type{}, std::true_type{});
+      step(std::false_type{}, std::false_type{});
     }
     {
       int tm, tn;
@@ -546,12 +610,15 @@ void gemm_tiled_kernel(GemmParams p) {
       if (EPI == kEpiPartial) {
         store_partial(m0, n0, c_split);
       } else {
-        const bool interior = (m0 + BM <= p.M) && (n0 + BN <= p.N) && ((p.ldc & 3) == 0) &&
-                              ((reinterpret_cast<uintptr_t>(p.c) & 7) == 0);
-        if (interior) epilogue(m0, n0, std::true_type{});
-        else epilogue(m0, n0, std::false_type{});
+        // sb already names the next step's stage; the one before it held this tile's last step
+        uint8_t* free_b = lds + LDS_B0 + ((sb + kStagesB - 1) % kStagesB) * STAGE_B;
+        const bool interior = (m0 + BM <= p.M) && (n0 + BN <= p.N);
+        const uintptr_t c_bits = reinterpret_cast<uintptr_t>(p.c) | (uintptr_t)(p.ldc * 2);
+        if (interior && (c_bits & 15) == 0) epilogue(m0, n0, std::true_type{}, free_b);
+        else epilogue(m0, n0, std::false_type{}, free_b);
       }
     }
+    read_first_half();  // of the next item's first step (landed before this item's last barrier)
   }
   __builtin_amdgcn_s_waitcnt(0x0070);  // the trailing dummy loads must land before LDS is released
 }
