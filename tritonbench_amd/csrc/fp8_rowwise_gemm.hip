@@ -353,10 +353,12 @@ void gemm_tiled_kernel(GemmParams p) {
     }
   };
   // Per half step: NMFMA MFMAs, NREAD LDS reads, A_GROUPS or B_GROUPS global->LDS loads, the
-  // memory instructions spread evenly behind the MFMAs (slot t gets reads [t*RPS, (t+1)*RPS)
-  // and load l when l*NMFMA/GROUPS == t).
+  // memory instructions placed behind the MFMAs: load l in slot l*NMFMA/GROUPS, the reads RPS
+  // per slot in the first half of the slots. The reads have then returned while the last
+  // MFMAs still execute, so the wait at the end of the half step (for the barrier, or for
+  // the fragments of the next half) costs the matrix pipe nothing.
   constexpr int NMFMA = MT * NT, NREAD = 2 * (MT + NT);
-  constexpr int RPS = (NREAD + NMFMA - 1) / NMFMA;
+  constexpr int RPS = (NREAD + NMFMA / 2 - 1) / (NMFMA / 2);
   static_assert(A_GROUPS <= NMFMA && B_GROUPS <= NMFMA, "at most one load slot per MFMA");
 
   // ---- prologue: A(0) B(0) A(1) B(1) in flight, first fragments in registers
