@@ -359,6 +359,44 @@ def test_quantiser_bf16_bit_exact(gpu_device, rows, cols):
     assert torch.equal(inv.cpu().view(torch.int32), want_inv.view(torch.int32))
 
 
+def test_quantiser_rounding_at_every_code_boundary(gpu_device):
+    # every finite e4m3fn value, every midpoint between neighbours (the ties) and the fp32
+    # numbers just below and above each midpoint, with 448 as the row maximum so the scale is 1:
+    # pins the conversion instruction's rounding against the oracle's cast code by code
+    t = np.sort(np.unique(e4m3.decode_table()[np.isfinite(e4m3.decode_table())].astype(np.float32)))
+    mids = ((t[:-1].astype(np.float64) + t[1:].astype(np.float64)) / 2).astype(np.float32)
+    vals = np.concatenate([t, mids, np.nextafter(mids, np.float32(-np.inf)), np.nextafter(mids, np.float32(np.inf)),
+                           np.float32([2.0 ** -10, 2.0 ** -11, 3 * 2.0 ** -11, 1e-30, -1e-30])])
+    for amax in (448.0, 1.0, 0.013):  # other row maxima move the same grid through other scales
+        row = (vals.astype(np.float64) * amax / 448.0).astype(np.float32)
+        pad = (-len(row)) % 4
+        x = torch.from_numpy(np.concatenate([row, np.zeros(pad, np.float32)])).reshape(1, -1)
+        want_q, want_inv = orc.fp8_row_quantize(x)
+        xq, inv = ops.fp8_row_quantize(x.to(gpu_device))
+        assert torch.equal(xq.cpu().view(torch.uint8), want_q.view(torch.uint8))
+        assert torch.equal(inv.cpu().view(torch.int32), want_inv.view(torch.int32))
+        xb = x.to(torch.bfloat16)
+        xb = torch.cat([xb, torch.zeros(1, (-xb.shape[1]) % 8, dtype=torch.bfloat16)], dim=1)
+        want_q, want_inv = orc.fp8_row_quantize(xb)
+        xq, inv = ops.fp8_row_quantize(xb.to(gpu_device))
+        assert torch.equal(xq.cpu().view(torch.uint8), want_q.view(torch.uint8))
+        assert torch.equal(inv.cpu().view(torch.int32), want_inv.view(torch.int32))
+
+
+@pytest.mark.parametrize("dtype,rows,cols,width", [(torch.float32, 3, 20000, 20000), (torch.bfloat16, 2, 20480, 20480),
+                                                     (torch.float32, 40, 1024, 1040), (torch.bfloat16, 40, 1000, 1024),
+                                                     (torch.float32, 6, 1002, 1003)])
+def test_quantiser_long_rows_and_strides(gpu_device, dtype, rows, cols, width):
+    # rows longer than the register cache of the vector kernel, row strides wider than the
+    # row (vector and scalar kernels), untouched bytes beyond each quantised row
+    buf = orc.randn_f32(rows, width, 1.0, seed=cols).to(dtype)
+    x = buf[:, :cols]
+    want_q, want_inv = orc.fp8_row_quantize(x.contiguous())
+    xq, inv = ops.fp8_row_quantize(buf.to(gpu_device)[:, :cols])
+    assert torch.equal(xq.cpu().view(torch.uint8), want_q.view(torch.uint8))
+    assert torch.equal(inv.cpu().view(torch.int32), want_inv.view(torch.int32))
+
+
 def test_quantiser_special_rows(gpu_device):
     x = torch.zeros(4, 64)
     x[1, 5] = 1e-20

@@ -911,6 +911,129 @@ __global__ __launch_bounds__(256) void quantize_rows_kernel(const SrcT* x, uint8
   }
 }
 
+// Vector form of the quantiser for 16-byte aligned rows: one workgroup per row, every lane
+// moves 16 source bytes per load (a wave-wide load covers whole lines). The first CACHE
+// chunks a lane reads stay in registers between the amax pass and the convert pass, so rows
+// of up to THREADS*CACHE chunks are read from memory once; the rest of a longer row is read
+// again (from cache). The e4m3fn rounding is done by the gfx950 pack-convert instruction
+// (OCP format, round to nearest even) on values already clamped to +-448.
+template <typename SrcT>
+struct VecTraits;
+template <>
+struct VecTraits<float> {
+  static constexpr int EPV = 4;  // elements per 16-byte chunk
+  static __device__ __forceinline__ void unpack(const v4i& c, float (&f)[4]) {
+#pragma unroll
+    for (int e = 0; e < 4; ++e) f[e] = __int_as_float(c[e]);
+  }
+};
+template <>
+struct VecTraits<uint16_t> {
+  static constexpr int EPV = 8;
+  static __device__ __forceinline__ void unpack(const v4i& c, float (&f)[8]) {
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      f[2 * e] = __uint_as_float((uint32_t)c[e] << 16);
+      f[2 * e + 1] = __uint_as_float((uint32_t)c[e] & 0xffff0000u);
+    }
+  }
+};
+
+template <typename SrcT, int CACHE, int THREADS>
+__global__ __launch_bounds__(THREADS) void quantize_rows_vec_kernel(const SrcT* x, uint8_t* xq,
+                                                                float* inv_scale, int K, long ldx,
+                                                                long ldq) {
+  using T = SrcTraits<SrcT>;
+  using V = VecTraits<SrcT>;
+  constexpr int EPV = V::EPV;
+  __shared__ float wave_max[THREADS / 64];
+  const long row = blockIdx.x;
+  const v4i* xr = (const v4i*)(x + row * ldx);
+  uint8_t* qr = xq + row * ldq;
+  const int nchunks = K / EPV;
+  const int tid = threadIdx.x;
+
+  v4i cache[CACHE];
+  float amax = 0.0f;
+  auto fold = [&](const v4i& c) {
+    float f[EPV];
+    V::unpack(c, f);
+#pragma unroll
+    for (int e = 0; e < EPV; ++e) amax = fmaxf(amax, fabsf(f[e]));
+  };
+#pragma unroll
+  for (int i = 0; i < CACHE; ++i) {
+    // past the row's end a lane re-reads the last chunk: harmless for the maximum, never
+    // stored, and it keeps the loads free of branches
+    cache[i] = __builtin_nontemporal_load(xr + min(tid + THREADS * i, nchunks - 1));
+  }
+#pragma unroll
+  for (int i = 0; i < CACHE; ++i) fold(cache[i]);
+  for (int c = tid + THREADS * CACHE; c < nchunks; c += THREADS) fold(xr[c]);
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) amax = fmaxf(amax, __shfl_xor(amax, o));
+  if ((tid & 63) == 0) wave_max[tid >> 6] = amax;
+  __syncthreads();
+#pragma unroll
+  for (int w = 0; w < THREADS / 64; ++w) amax = fmaxf(amax, wave_max[w]);
+
+  const float recip = T::round(1.0f / fmaxf(amax, T::round(1e-12f)));
+  const float scale = T::round(recip * 448.0f);
+  if (tid == 0) inv_scale[row] = T::round(1.0f / scale);
+
+  auto convert = [&](const v4i& src, uint32_t (&out)[EPV / 4]) {
+    float f[EPV];
+    V::unpack(src, f);
+#pragma unroll
+    for (int e = 0; e < EPV; ++e) f[e] = fminf(fmaxf(T::round(f[e] * scale), -448.0f), 448.0f);
+#pragma unroll
+    for (int w = 0; w < EPV / 4; ++w) {
+      int packed = __builtin_amdgcn_cvt_pk_fp8_f32(f[4 * w], f[4 * w + 1], 0, false);
+      packed = __builtin_amdgcn_cvt_pk_fp8_f32(f[4 * w + 2], f[4 * w + 3], packed, true);
+      out[w] = (uint32_t)packed;
+    }
+  };
+  auto convert_store = [&](const v4i& src, int c) {
+    uint32_t out[EPV / 4];
+    convert(src, out);
+    if (EPV == 4) *(uint32_t*)(qr + (size_t)c * 4) = out[0];
+    else *(v2u*)(qr + (size_t)c * 8) = (v2u){out[0], out[EPV / 4 - 1]};
+  };
+  // A chunk turns into EPV output bytes per lane (4 or 8): too little per store instruction.
+  // BATCH = 16 / EPV consecutive rounds of the cached chunks are therefore gathered through
+  // a wave-private LDS strip (LDS executes a wave's operations in order: no barrier) and
+  // leave as one 16-byte store per lane, BATCH runs of 1024 / BATCH contiguous bytes each.
+  constexpr int BATCH = 16 / EPV;
+  static_assert(CACHE % BATCH == 0, "cached rounds must split into whole batches");
+  __shared__ __attribute__((aligned(16))) uint8_t strip[THREADS / 64][1024];
+  uint8_t* mine = strip[tid >> 6];
+  const int lane = tid & 63;
+  constexpr int LPR = 64 / BATCH;  // lanes that store one round's bytes of this wave
+#pragma unroll
+  for (int i0 = 0; i0 < CACHE; i0 += BATCH) {
+    if (THREADS * (i0 + BATCH) <= nchunks) {  // uniform: every lane of every wave has all BATCH rounds
+#pragma unroll
+      for (int b = 0; b < BATCH; ++b) {
+        uint32_t out[EPV / 4];
+        convert(cache[i0 + b], out);
+        if (EPV == 4) *(uint32_t*)(mine + b * 256 + lane * 4) = out[0];
+        else *(v2u*)(mine + b * 512 + lane * 8) = (v2u){out[0], out[EPV / 4 - 1]};
+      }
+      const int b = lane / LPR, piece = lane % LPR;
+      const v4i bytes = *(const v4i*)(mine + lane * 16);
+      // round i0+b, this wave's 64 chunks start at chunk THREADS*(i0+b) + 64*wave
+      *(v4i*)(qr + ((size_t)THREADS * (i0 + b) + (tid & ~63)) * EPV + piece * 16) = bytes;
+    } else {
+#pragma unroll
+      for (int b = 0; b < BATCH; ++b) {
+        const int c = tid + THREADS * (i0 + b);
+        if (c < nchunks) convert_store(cache[i0 + b], c);
+      }
+    }
+  }
+  for (int c = tid + THREADS * CACHE; c < nchunks; c += THREADS) convert_store(xr[c], c);
+}
+
 // ------------------------------------------------------------------------------------
 // Host side
 // ------------------------------------------------------------------------------------
@@ -1179,7 +1302,22 @@ int mi355x_fp8_rowwise_quantize(const void* x, int src_type, void* xq, float* in
   if (R < 1 || K < 1 || ldx < K || ldq < K) return fail(MI355X_FP8_EINVAL, "bad shape or leading dimension");
   if (R > INT32_MAX || K > INT32_MAX) return fail(MI355X_FP8_ENOTSUP, "dimension exceeds 2^31-1");
   hipStream_t s = (hipStream_t)stream;
-  if (src_type == MI355X_FP8_SRC_F32) {
+  // source and destination rows that start 16-byte aligned and hold whole 16-byte source
+  // chunks take the vector kernel
+  const int esz = src_type == MI355X_FP8_SRC_BF16 ? 2 : 4;
+  const int epv = 16 / esz;
+  const bool vec = (reinterpret_cast<uintptr_t>(x) & 15) == 0 && (ldx * esz) % 16 == 0 && K % epv == 0 &&
+                   (reinterpret_cast<uintptr_t>(xq) & 15) == 0 && ldq % 16 == 0;
+  const bool long_row = K / epv > 8 * 256;  // more chunks than 256 lanes keep in registers
+  if (vec && src_type == MI355X_FP8_SRC_F32) {
+    auto kern = long_row ? quantize_rows_vec_kernel<float, 8, 1024> : quantize_rows_vec_kernel<float, 8, 256>;
+    hipLaunchKernelGGL(kern, dim3((unsigned)R), dim3(long_row ? 1024 : 256), 0, s, (const float*)x,
+                       (uint8_t*)xq, inv_scale, (int)K, (long)ldx, (long)ldq);
+  } else if (vec && src_type == MI355X_FP8_SRC_BF16) {
+    auto kern = long_row ? quantize_rows_vec_kernel<uint16_t, 8, 1024> : quantize_rows_vec_kernel<uint16_t, 8, 256>;
+    hipLaunchKernelGGL(kern, dim3((unsigned)R), dim3(long_row ? 1024 : 256), 0, s,
+                       (const uint16_t*)x, (uint8_t*)xq, inv_scale, (int)K, (long)ldx, (long)ldq);
+  } else if (src_type == MI355X_FP8_SRC_F32) {
     hipLaunchKernelGGL(quantize_rows_kernel<float>, dim3((unsigned)R), dim3(256), 0, s, (const float*)x,
                        (uint8_t*)xq, inv_scale, (int)K, (long)ldx, (long)ldq);
   } else if (src_type == MI355X_FP8_SRC_BF16) {
