@@ -727,6 +727,25 @@ __global__ __launch_bounds__(KW * 64) void gemm_skinny_kernel(GemmParams p) {
 #pragma unroll
     for (int u = 0; u < MT; ++u) acc[t][u] = (v4f){0.f, 0.f, 0.f, 0.f};
 
+  // The lanes that will finish an output quad (one per lane of each 16x16 result) fetch its
+  // scales and bias now, so that their latency is not left over at the end of the kernel.
+  // Lane layout of a 16x16 result: m = u*16 + lane%16, n = n0 + t*16 + 4*(lane/16) + e.
+  static_assert(NTW * MT * 64 <= KW * 64, "one finishing lane per output quad");
+  const bool finisher = threadIdx.x < NTW * MT * 64;
+  const int fin_tu = threadIdx.x >> 6;
+  const int fin_m = (fin_tu % MT) * 16 + (lane & 15);
+  const int fin_n = n0 + (fin_tu / MT) * 16 + 4 * (lane >> 4);
+  float fin_sa = 0.f, fin_sb[4] = {0.f, 0.f, 0.f, 0.f}, fin_bias[4] = {0.f, 0.f, 0.f, 0.f};
+  if (finisher) {
+    fin_sa = p.a_scale[min(fin_m, p.M - 1)];
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      const int ne = min(fin_n + e, p.N - 1);
+      fin_sb[e] = p.b_scale[ne];
+      if (p.bias) fin_bias[e] = bf16_to_f32(p.bias[ne]);
+    }
+  }
+
   // DEPTH register sets, one per step in flight
   v4i land[DEPTH][NTILE][2];
   auto fetch = [&](int i, v4i (&dst)[NTILE][2]) {
@@ -810,33 +829,25 @@ __global__ __launch_bounds__(KW * 64) void gemm_skinny_kernel(GemmParams p) {
     for (int u = 0; u < MT; ++u) mine[(t * MT + u) * 64 + lane] = acc[t][u];
   __syncthreads();
 
-  // Lane layout of a 16x16 result: m = u*16 + lane%16, n = n0 + t*16 + 4*(lane/16) + e.
-  for (int idx = threadIdx.x; idx < NTW * MT * 64; idx += KW * 64) {
-    const int tu = idx >> 6, l = idx & 63;
-    const int t = tu / MT, u = tu % MT;
-    v4f sum = ((const v4f*)lds)[tu * 64 + l];
+  if (finisher && fin_m < p.M && fin_n < p.N) {
+    v4f sum = ((const v4f*)lds)[fin_tu * 64 + lane];
 #pragma unroll
-    for (int w = 1; w < KW; ++w) sum += ((const v4f*)(lds + w * BUF))[tu * 64 + l];
-    const int m = u * 16 + (l & 15);
-    const int n = n0 + t * 16 + 4 * (l >> 4);
-    if (m >= p.M || n >= p.N) continue;
-    const float sa_m = p.a_scale[m];
+    for (int w = 1; w < KW; ++w) sum += ((const v4f*)(lds + w * BUF))[fin_tu * 64 + lane];
     float r[4];
 #pragma unroll
     for (int e = 0; e < 4; ++e) {
-      const int ne = min(n + e, p.N - 1);
-      r[e] = sum[e] * sa_m * p.b_scale[ne];
-      if (p.bias) r[e] += bf16_to_f32(p.bias[ne]);
+      r[e] = sum[e] * fin_sa * fin_sb[e];
+      if (p.bias) r[e] += fin_bias[e];
     }
     const uint32_t lo = pack_bf16x2(r[0], r[1]), hi = pack_bf16x2(r[2], r[3]);
-    uint16_t* dst = p.c + (size_t)m * p.ldc + n;
-    if (n + 3 < p.N && ((p.ldc & 3) == 0) && ((reinterpret_cast<uintptr_t>(p.c) & 7) == 0)) {
+    uint16_t* dst = p.c + (size_t)fin_m * p.ldc + fin_n;
+    if (fin_n + 3 < p.N && ((p.ldc & 3) == 0) && ((reinterpret_cast<uintptr_t>(p.c) & 7) == 0)) {
       *(v2u*)dst = (v2u){lo, hi};
     } else {
       dst[0] = (uint16_t)lo;
-      if (n + 1 < p.N) dst[1] = (uint16_t)(lo >> 16);
-      if (n + 2 < p.N) dst[2] = (uint16_t)hi;
-      if (n + 3 < p.N) dst[3] = (uint16_t)(hi >> 16);
+      if (fin_n + 1 < p.N) dst[1] = (uint16_t)(lo >> 16);
+      if (fin_n + 2 < p.N) dst[2] = (uint16_t)hi;
+      if (fin_n + 3 < p.N) dst[3] = (uint16_t)(hi >> 16);
     }
   }
 }

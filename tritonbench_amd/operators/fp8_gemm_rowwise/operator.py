@@ -146,7 +146,8 @@ class Operator(BenchmarkOperator):
         if not xq.is_cuda:
             raise NotImplementedError("the MI355X backend needs device tensors (run with --device cuda)")
         out = torch.empty((xq.shape[0], wq.shape[0]), dtype=torch.bfloat16, device=xq.device)
-        return lambda: ops.fp8_gemm_rowwise(xq, wq, x_scale, w_scale, bias=bias, out=out)
+        workspace = ops.gemm_workspace(xq.shape[0], wq.shape[0], xq.shape[1], xq.device)
+        return lambda: ops.fp8_gemm_rowwise(xq, wq, x_scale, w_scale, bias=bias, out=out, workspace=workspace)
 
     @register_benchmark(baseline=True, label="torch_cpu_ref")
     def _torch_dequant_cpu(self, xq, wq, x_scale, w_scale, bias) -> Callable:

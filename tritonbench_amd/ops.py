@@ -29,6 +29,13 @@ def select_variant(m: int, n: int, k: int) -> int:
     return v
 
 
+def gemm_workspace(m: int, n: int, k: int, device, variant: int = _lib.VARIANT_AUTO) -> Optional[torch.Tensor]:
+    """Device workspace the plan for this shape wants (fp32 split-K partial sums), or None.
+    Allocate it once and pass it as `workspace=` to keep allocation out of repeated calls."""
+    nbytes = _lib.load().mi355x_fp8_rowwise_workspace_bytes(m, n, k, variant)
+    return torch.empty(nbytes, dtype=torch.uint8, device=device) if nbytes else None
+
+
 def fp8_gemm_rowwise(
     xq: torch.Tensor,
     wq: torch.Tensor,
@@ -37,12 +44,16 @@ def fp8_gemm_rowwise(
     bias: Optional[torch.Tensor] = None,
     out: Optional[torch.Tensor] = None,
     variant: int = _lib.VARIANT_AUTO,
+    workspace: Optional[torch.Tensor] = None,
 ) -> torch.Tensor:
     """bf16 [M,N] = ((xq @ wq.T) * x_scale[:,None] * w_scale[None,:] + bias).
 
     Same operands as the callables of tritonbench/operators/fp8_gemm_rowwise/operator.py:187-217:
     xq [M,K] and wq [N,K] float8_e4m3fn, x_scale [M] and w_scale [N] float32, bias [N]
-    bfloat16 or None. Only enqueues work on the current stream (graph-capturable).
+    bfloat16 or None. Only enqueues work on the current stream (graph-capturable). Shapes
+    whose plan splits K need a workspace: pass one from gemm_workspace(), or leave it to this
+    call (a torch.empty per call; too small a workspace makes the library run a plan that
+    needs none).
     """
     lib = _lib.load()
     for t, name in ((xq, "xq"), (wq, "wq"), (x_scale, "x_scale"), (w_scale, "w_scale")):
@@ -73,10 +84,14 @@ def fp8_gemm_rowwise(
         _require_gpu(out, "out")
         if out.dtype != torch.bfloat16 or tuple(out.shape) != (m, n) or out.stride(1) != 1:
             raise ValueError("out must be bfloat16 [M,N] with unit column stride")
-    ws_bytes = lib.mi355x_fp8_rowwise_workspace_bytes(m, n, k, variant)
-    ws = None
-    if ws_bytes:
-        ws = torch.empty(ws_bytes, dtype=torch.uint8, device=xq.device)
+    if workspace is not None:
+        _require_gpu(workspace, "workspace")
+        if not workspace.is_contiguous():
+            raise ValueError("workspace must be contiguous")
+        ws, ws_bytes = workspace, workspace.numel() * workspace.element_size()
+    else:
+        ws_bytes = lib.mi355x_fp8_rowwise_workspace_bytes(m, n, k, variant)
+        ws = torch.empty(ws_bytes, dtype=torch.uint8, device=xq.device) if ws_bytes else None
     st = lib.mi355x_fp8_rowwise_gemm(
         xq.data_ptr(), wq.data_ptr(), x_scale.data_ptr(), w_scale.data_ptr(), bias_ptr,
         out.data_ptr(), m, n, k, xq.stride(0), wq.stride(0), out.stride(0),

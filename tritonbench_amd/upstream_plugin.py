@@ -28,7 +28,8 @@ def _hip_mi355x(self, xq, wq, x_scale, w_scale, bias) -> Callable:
     """Backend method: same signature as the upstream `_triton` / `_cutlass_or_ck`
     methods (operator.py:187-217), returns a zero-argument callable."""
     out = torch.empty((xq.shape[0], wq.shape[0]), dtype=torch.bfloat16, device=xq.device)
-    return lambda: ops.fp8_gemm_rowwise(xq, wq, x_scale, w_scale, bias=bias, out=out)
+    workspace = ops.gemm_workspace(xq.shape[0], wq.shape[0], xq.shape[1], xq.device)
+    return lambda: ops.fp8_gemm_rowwise(xq, wq, x_scale, w_scale, bias=bias, out=out, workspace=workspace)
 
 
 def register(operator_cls, baseline: bool = False) -> None:
