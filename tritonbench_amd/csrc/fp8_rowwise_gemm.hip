@@ -6,15 +6,20 @@
 // on the gfx950 f8f6f4 MFMA instructions (full FP8 rate) with fp32 accumulation; scales and
 // bias are applied in fp32 to the accumulator and the result is rounded to bf16 once.
 //
-// Two kernel families:
-//   gemm_tiled_kernel   persistent workgroups, BM x BN x 128 tiles staged global->LDS with
-//                       direct-to-LDS loads into two swizzled stages, 32x32x64 MFMA.
-//   gemm_skinny_kernel  M <= 64: every workgroup owns 16 rows of B and all of K, its waves
-//                       split K between them and reduce through LDS; B is streamed once.
+// Kernels:
+//   gemm_tiled_kernel        persistent workgroups walk (split, tile) work items; BM x BN x 128
+//                            steps staged global->LDS with direct-to-LDS loads into swizzled
+//                            rings (2 stages of A, 3 of B), 32x32x64 MFMA, epilogue turned
+//                            through LDS into 16-byte row stores. 256x256 and 128x128 tiles.
+//   splitk_finalize_kernel   adds the fp32 partial sums of a split-K launch, applies scales/bias.
+//   gemm_skinny_kernel       M <= 64: every workgroup owns 16 rows of B and all of K, its waves
+//                            split K between them and reduce through LDS; B is streamed once.
+//   quantize_rows_*_kernel   row-wise e4m3fn quantiser (amax, scale, convert), one row per workgroup.
 //
 // Operand roles inside the MFMA are swapped on purpose (rows of B feed the instruction's
 // "A" port, rows of A its "B" port) so each lane ends up holding 4 consecutive columns n of
-// one output row m and can store them as one 8-byte write.
+// one output row m (16 bytes of fp32 for the epilogue's LDS turn, 8 bytes of bf16 in the
+// skinny kernel's direct stores).
 
 #include <hip/hip_runtime.h>
 #include <stdint.h>
@@ -671,8 +676,8 @@ __global__ __launch_bounds__(256) void splitk_finalize_kernel(GemmParams p) {
 // Skinny kernel (M <= 16*MT, HBM-bound): B is streamed exactly once and nothing is reused, so
 // what matters is whole-line coalesced loads and as many bytes in flight as a plain copy has.
 //
-// A workgroup owns 16*NTW rows of B and all of K; its 16 waves split K between them in
-// interleaved 128-byte steps (wave w takes steps w, w+16, ...: the workgroup reads 2 KB runs
+// A workgroup owns 16*NTW rows of B and all of K; its KW waves split K between them in
+// interleaved 128-byte steps (wave w takes steps w, w+KW, ...: the workgroup reads KW*128-byte runs
 // of every row). Registers are the landing zone: a wave keeps DEPTH steps of loads in flight
 // (16 bytes per lane, 8 lanes per row, so every wave-wide load moves 8 whole 128-byte lines;
 // letting each MFMA lane fetch its own row instead costs the memory pipeline four times the
