@@ -106,6 +106,34 @@ int mi355x_fp8_rowwise_gemm(const void* a, const void* b,
                             int variant, void* stream);
 
 /*
+ * Grouped form (mixture-of-experts layers): A and C are G row blocks stacked in one
+ * matrix, block g holding m_sizes[g] rows; block g is multiplied with rows
+ * [g*N, (g+1)*N) of B:
+ *
+ *   C[r, n] = bf16( (sum_k A[r,k] * B[g*N + n, k]) * a_scale[r] * b_scale[g*N + n] )   r in block g
+ *
+ * Replaces the timed callables of
+ * tritonbench/operators/fp8_gemm_rowwise_grouped/operator.py:400-424
+ * (grouped_gemm_fp8_rowwise(group_A, group_B, m_sizes, a_scale, b_scale)) and :426-455.
+ *
+ *   a        e4m3fn [M, K]                      b        e4m3fn [G*N, K]
+ *   a_scale  f32 [M]                            b_scale  f32 [G*N], 16-byte aligned
+ *   m_sizes  int32 [G] in DEVICE memory         c        bf16 [M, N]
+ *
+ * The sizes are read by the kernel, not by the host (no synchronisation): negative sizes
+ * count as 0 and rows past M are cut off, so the kernel never leaves A or C whatever the
+ * sizes say. Rows of C past the sum of the sizes are left untouched. `tile_config` is -1
+ * (the library picks from M / G) or one of the tile configurations listed above.
+ * Same alignment requirements as mi355x_fp8_rowwise_gemm.
+ */
+int mi355x_fp8_rowwise_grouped_gemm(const void* a, const void* b,
+                                    const float* a_scale, const float* b_scale,
+                                    const int32_t* m_sizes, void* c,
+                                    int64_t G, int64_t M, int64_t N, int64_t K,
+                                    int64_t lda, int64_t ldb, int64_t ldc,
+                                    int tile_config, void* stream);
+
+/*
  * Row-wise e4m3fn quantiser, replacing fp8_row_quantize (operator.py:136-145):
  *   amax[r]      = max_k |x[r,k]|
  *   scale[r]     = fl(fl(1 / max(amax[r], 1e-12)) * 448)   (how PyTorch evaluates 448 / tensor)

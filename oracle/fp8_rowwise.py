@@ -176,6 +176,39 @@ def make_inputs(m: int, n: int, k: int, sigma: float = 1.0, bias: bool = False):
 
 
 # The five workload families the parity and bench code iterate over.
+def grouped_dequant_matmul(xq, wq, m_sizes, x_scale, w_scale):
+    """Grouped form on the CPU: rows of group g (m_sizes[g] consecutive rows, in order) times
+    wq[g*N:(g+1)*N].T with both scales, fp32 dequantise + matmul, one bf16 rounding; rows past
+    sum(m_sizes) are zero. Follows the per-group expression of the reference's torch baseline,
+    tritonbench/operators/fp8_gemm_rowwise_grouped/operator.py:689-699, with the group
+    boundaries taken from m_sizes as its Triton and CK backends do (:400-455); the random
+    boundaries the reference baseline draws at :676-686 are a quirk of that baseline and are
+    not restated."""
+    sizes = [int(v) for v in m_sizes]
+    g = len(sizes)
+    m, k = xq.shape
+    n = wq.shape[0] // g
+    out = torch.zeros((m, n), dtype=torch.bfloat16)
+    start = 0
+    for i, mg in enumerate(sizes):
+        end = min(start + max(mg, 0), m)
+        if end > start:
+            out[start:end] = dequant_matmul(xq[start:end], wq[i * n:(i + 1) * n], x_scale[start:end],
+                                            w_scale[i * n:(i + 1) * n])
+        start = end
+    return out
+
+
+def make_grouped_inputs(g, m, n, k, sigma=1.0, sizes=None, seed_tag=0):
+    """Seeded operands of the grouped form: A [M,K], B [G*N,K] quantised row-wise, m_sizes int32
+    [G] (equal split M // G as at operator.py:563-565 unless `sizes` is given)."""
+    xq, xs = fp8_row_quantize(randn_f32(m, k, sigma, seed=MAIN_RANDOM_SEED + 17 * m + k + seed_tag))
+    wq, ws = fp8_row_quantize(randn_f32(g * n, k, sigma, seed=MAIN_RANDOM_SEED + 31 * n + k + g + seed_tag))
+    if sizes is None:
+        sizes = [m // g] * g
+    return xq, wq, torch.tensor(sizes, dtype=torch.int32), xs, ws
+
+
 LLAMA3_70B_NK = {"qkv": (10240, 8192), "o_proj": (8192, 8192), "gate_up": (57344, 8192), "down": (8192, 28672)}
 LLAMA3_70B_M = (1, 32, 128, 1024, 4096)
 CONFIGS = {

@@ -1,0 +1,166 @@
+"""Parity of the grouped HIP path (through the C ABI) with the CPU oracle. Needs an MI355X."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import e4m3
+from oracle import fp8_rowwise as orc
+from tritonbench_amd import _lib, ops
+
+pytestmark = pytest.mark.gpu
+
+RTOL = 1e-2  # the tolerance the path is specified to
+ATOL = 1e-2
+
+
+def _bits(t):
+    return t.view(torch.int16).cpu().numpy().view(np.uint16)
+
+
+def _run(dev, xq, wq, ms, xs, ws, tile_config=-1, out=None):
+    res = ops.fp8_gemm_rowwise_grouped(xq.to(dev), wq.to(dev), ms.to(dev), xs.to(dev), ws.to(dev), out=out,
+                                       tile_config=tile_config)
+    torch.cuda.synchronize()
+    return res.cpu()
+
+
+def _check(out, want, operands=None):
+    torch.testing.assert_close(out, want, rtol=RTOL, atol=ATOL)
+    if operands is None:
+        return
+    # beyond rtol/atol: within 1 bf16 ulp of the float64 value plus the slack any fp32
+    # accumulation order is entitled to (keeps parity meaningful where |C| << atol)
+    xq, wq, ms, xs, ws = operands
+    a = e4m3.decode(xq.view(torch.uint8).numpy()).astype(np.float64)
+    b = e4m3.decode(wq.view(torch.uint8).numpy()).astype(np.float64)
+    sa, sb = xs.numpy().astype(np.float64), ws.numpy().astype(np.float64)
+    n, k = out.shape[1], a.shape[1]
+    got = out.float().numpy().astype(np.float64)
+    start = 0
+    for g, mg in enumerate(int(v) for v in ms):
+        end = min(start + max(mg, 0), got.shape[0])
+        if end > start:
+            bg, sg = b[g * n:(g + 1) * n], sb[g * n:(g + 1) * n]
+            exact = (a[start:end] @ bg.T) * sa[start:end, None] * sg[None, :]
+            slack = (np.abs(a[start:end]) @ np.abs(bg).T) * sa[start:end, None] * sg[None, :] * k * 2.0 ** -24
+            ulp = 2.0 ** (np.floor(np.log2(np.maximum(np.abs(exact), 2.0 ** -126))) - 7)
+            assert np.all(np.abs(got[start:end] - exact) <= ulp + slack)
+        start = end
+
+
+CASES = [
+    # g, m, n, k, sizes (None = equal split as the reference's input generator makes them)
+    (2, 1024, 1024, 1024, None),
+    (4, 2048, 1024, 1024, None),
+    (4, 512, 384, 272, None),                      # K tail
+    (3, 700, 520, 1040, [300, 0, 400]),            # empty group, ragged tiles in M and N
+    (5, 1000, 260, 512, [1, 255, 256, 257, 231]),  # sizes around the tile edges
+    (8, 640, 128, 256, [80] * 8),                  # many small groups
+    (2, 300, 130, 128, [100, 150]),                # rows past the sum stay untouched; N % 4 != 0
+    (6, 900, 256, 384, [0, 0, 500, 0, 400, 0]),    # empty groups first, between and last
+]
+
+
+@pytest.mark.parametrize("g,m,n,k,sizes", CASES)
+@pytest.mark.parametrize("tile_config", [-1] + list(range(_lib.NUM_TILE_CONFIGS)))
+def test_grouped_against_oracle(gpu_device, g, m, n, k, sizes, tile_config):
+    print(f"case g={g} m={m} n={n} k={k} sizes={sizes} tile_config={tile_config}", flush=True)
+    xq, wq, ms, xs, ws = orc.make_grouped_inputs(g, m, n, k, sizes=sizes)
+    want = orc.grouped_dequant_matmul(xq, wq, ms, xs, ws)
+    covered = min(int(ms.clamp(min=0).sum()), m)
+    canvas = torch.full((m, n), -77.0, dtype=torch.bfloat16, device=gpu_device)
+    out = _run(gpu_device, xq, wq, ms, xs, ws, tile_config, out=canvas)
+    _check(out[:covered], want[:covered], (xq, wq, ms, xs, ws))
+    assert torch.all(out[covered:] == -77.0)  # rows no group owns are not written
+
+
+@pytest.mark.parametrize("tile_config", range(_lib.NUM_TILE_CONFIGS))
+def test_grouped_sizes_that_lie_are_cut_off_inside_the_matrices(gpu_device, tile_config):
+    # the kernel reads the sizes, the host never does: negative entries count as empty and the
+    # running sum stops at M, so nothing outside A and C is touched whatever the entries say
+    g, m, n, k = 4, 520, 256, 256
+    xq, wq, _, xs, ws = orc.make_grouped_inputs(g, m, n, k)
+    ms = torch.tensor([200, -5, 10000, 300], dtype=torch.int32)
+    want = orc.grouped_dequant_matmul(xq, wq, ms, xs, ws)  # same rule: group 2 gets rows 200..519
+    buf = torch.full((m + 4, n), -77.0, dtype=torch.bfloat16, device=gpu_device)
+    ops.fp8_gemm_rowwise_grouped(xq.to(gpu_device), wq.to(gpu_device), ms.to(gpu_device), xs.to(gpu_device),
+                                 ws.to(gpu_device), out=buf[:m], tile_config=tile_config)
+    torch.cuda.synchronize()
+    _check(buf[:m].cpu(), want, (xq, wq, ms, xs, ws))
+    assert torch.all(buf[m:] == -77.0)
+
+
+@pytest.mark.parametrize("tile_config", range(_lib.NUM_TILE_CONFIGS))
+def test_grouped_exact_integer_case_is_bit_exact(gpu_device, tile_config):
+    rng = np.random.default_rng(21)
+    ints = np.array([0, 1, 2, 3, 4, -1, -2, -3, -4, 0.5, -0.5], dtype=np.float32)
+    g, n, k = 3, 200, 1040
+    sizes = [130, 257, 90]
+    m = sum(sizes)
+    a = rng.choice(ints, size=(m, k)).astype(np.float32)
+    b = rng.choice(ints, size=(g * n, k)).astype(np.float32)
+    out = _run(gpu_device, torch.from_numpy(a).to(torch.float8_e4m3fn), torch.from_numpy(b).to(torch.float8_e4m3fn),
+               torch.tensor(sizes, dtype=torch.int32), torch.ones(m), torch.ones(g * n), tile_config)
+    want = np.zeros((m, n), np.float64)
+    start = 0
+    for i, mg in enumerate(sizes):
+        want[start:start + mg] = a[start:start + mg].astype(np.float64) @ b[i * n:(i + 1) * n].astype(np.float64).T
+        start += mg
+    assert np.array_equal(_bits(out), orc.to_bf16_bits(want.astype(np.float32)))
+
+
+def test_grouped_with_one_group_equals_the_plain_kernel_bit_for_bit(gpu_device):
+    m, n, k = 600, 520, 768
+    xq, wq, ms, xs, ws = orc.make_grouped_inputs(1, m, n, k)
+    for cfg in range(_lib.NUM_TILE_CONFIGS):
+        grouped = _run(gpu_device, xq, wq, ms, xs, ws, cfg)
+        plain = ops.fp8_gemm_rowwise(xq.to(gpu_device), wq.to(gpu_device), xs.to(gpu_device), ws.to(gpu_device),
+                                     variant=_lib.tiled_variant(cfg, 1)).cpu()
+        assert torch.equal(grouped, plain)
+
+
+def test_grouped_graph_capture_replays_match_eager(gpu_device):
+    dev = gpu_device
+    xq, wq, ms, xs, ws = orc.make_grouped_inputs(4, 1024, 512, 640, sizes=[100, 400, 24, 500])
+    d = [t.to(dev) for t in (xq, wq, ms, xs, ws)]
+    eager = ops.fp8_gemm_rowwise_grouped(*d)
+    torch.cuda.synchronize()
+    out = torch.zeros_like(eager)
+    stream = torch.cuda.Stream()
+    with torch.cuda.stream(stream):
+        ops.fp8_gemm_rowwise_grouped(*d, out=out)
+        torch.cuda.synchronize()
+        g = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g, stream=stream):
+            for _ in range(3):
+                ops.fp8_gemm_rowwise_grouped(*d, out=out)
+        for _ in range(3):
+            out.zero_()
+            torch.cuda.synchronize()
+            g.replay()
+            torch.cuda.synchronize()
+            assert torch.equal(out, eager)
+    # new sizes in the same device tensor are picked up by the captured launch (the host never read them)
+    d[2].copy_(torch.tensor([500, 24, 400, 100], dtype=torch.int32))
+    want = orc.grouped_dequant_matmul(xq, wq, d[2].cpu(), xs, ws)
+    with torch.cuda.stream(stream):
+        out.zero_()
+        torch.cuda.synchronize()
+        g.replay()
+        torch.cuda.synchronize()
+    _check(out.cpu(), want)
+
+
+def test_grouped_invalid_arguments_raise(gpu_device):
+    dev = gpu_device
+    xq, wq, ms, xs, ws = (t.to(dev) for t in orc.make_grouped_inputs(2, 64, 32, 64))
+    with pytest.raises(ValueError, match="multiple"):
+        ops.fp8_gemm_rowwise_grouped(xq, wq[:-1], ms, xs, ws[:-1])
+    with pytest.raises(ValueError, match="int32"):
+        ops.fp8_gemm_rowwise_grouped(xq, wq, ms.to(torch.int64), xs, ws)
+    with pytest.raises(RuntimeError, match="no CPU fallback"):
+        ops.fp8_gemm_rowwise_grouped(xq, wq, ms.cpu(), xs, ws)
+    with pytest.raises(ValueError, match="tile configuration"):
+        ops.fp8_gemm_rowwise_grouped(xq, wq, ms, xs, ws, tile_config=_lib.NUM_TILE_CONFIGS)
+    with pytest.raises(NotImplementedError, match="multiple of 16"):
+        ops.fp8_gemm_rowwise_grouped(xq[:, :24], wq[:, :24], ms, xs, ws)

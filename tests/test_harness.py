@@ -303,3 +303,33 @@ def test_hip_backend_refuses_host_tensors():
         ops.fp8_gemm_rowwise(
             torch.zeros(16, 16).to(torch.float8_e4m3fn), torch.zeros(16, 16).to(torch.float8_e4m3fn),
             torch.ones(16), torch.ones(16))
+
+
+def test_grouped_operator_cpu_plumbing():
+    from tritonbench_amd.harness.loader import list_operators, load_opbench_by_name
+
+    assert "fp8_gemm_rowwise_grouped" in list_operators()
+    Op = load_opbench_by_name("fp8_gemm_rowwise_grouped")
+    args, extra = get_parser().parse_known_args(
+        ["--op", "fp8_gemm_rowwise_grouped", "--device", "cpu", "--m", "96", "--n", "64", "--k", "128",
+         "--group_size", "3", "--metrics", "latency,tflops,gbps", "--only", "_torch_dequant_cpu"])
+    op = Op(tb_args=args, extra_args=extra)
+    assert op.shapes == [(96, 64, 128)] and op.group_sizes == [3]
+    group_A, group_B, m_sizes, a_scale, b_scale = next(op.get_input_iter())
+    assert group_A.shape == (96, 128) and group_B.shape == (3 * 64, 128)
+    assert m_sizes.dtype == torch.int32 and m_sizes.tolist() == [32, 32, 32]
+    assert a_scale.shape == (96,) and b_scale.shape == (192,)
+    # the host baseline is the oracle's grouped product
+    from oracle import fp8_rowwise as orc
+    want = orc.grouped_dequant_matmul(group_A, group_B, m_sizes, a_scale, b_scale)
+    assert torch.equal(op._torch_dequant_cpu(group_A, group_B, m_sizes, a_scale, b_scale)(), want)
+    op.run(1, 2)
+    headers, table = op.output._table()
+    assert headers == ["(group_size, M, N, K)", "torch_cpu_ref-latency", "torch_cpu_ref-tflops", "torch_cpu_ref-gbps"]
+    assert table[0][0] == (3, 96, 64, 128)
+    lat = table[0][1].p50
+    assert table[0][2] == pytest.approx(2 * 96 * 64 * 128 / lat / 1e12 * 1e3)
+    assert table[0][3] == pytest.approx((96 * 128 + 3 * 64 * 128 + 2 * 96 * 64) / 1e9 / lat * 1e3)
+    assert REGISTERED_BENCHMARKS["fp8_gemm_rowwise_grouped"]["_hip_mi355x"].label == "hip_mi355x"
+    with pytest.raises((RuntimeError, NotImplementedError)):
+        op._hip_mi355x(group_A, group_B, m_sizes, a_scale, b_scale)()

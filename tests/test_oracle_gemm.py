@@ -162,3 +162,54 @@ def test_split_form_equals_dequant_matmul():
     rows = torch.tensor([0, 7, 39])
     part = orc.dequant_matmul_rows(orc.dequantize(xq[rows], xs[rows]), orc.dequantize(wq, ws), b)
     assert torch.equal(part, whole[rows])
+
+
+# ---- grouped form -------------------------------------------------------------------------
+def _grouped_bruteforce(xq, wq, sizes, xs, ws):
+    """Row by row in float64: the group of a row is found from the running sum of the sizes."""
+    a = e4m3.decode(xq.view(torch.uint8).numpy()).astype(np.float64)
+    b = e4m3.decode(wq.view(torch.uint8).numpy()).astype(np.float64)
+    m, n = a.shape[0], b.shape[0] // len(sizes)
+    out = np.zeros((m, n))
+    bounds = np.cumsum([0] + [max(int(s), 0) for s in sizes])
+    for r in range(m):
+        g = int(np.searchsorted(bounds, r, side="right")) - 1
+        if g >= len(sizes):
+            continue  # past the last group: stays zero
+        for c in range(n):
+            out[r, c] = np.dot(a[r], b[g * n + c]) * float(xs[r]) * float(ws[g * n + c])
+    return out
+
+
+@pytest.mark.parametrize("g,m,n,k,sizes", [
+    (2, 12, 5, 32, None), (3, 20, 7, 48, [5, 0, 9]), (4, 16, 3, 16, [1, 2, 3, 10]), (1, 9, 4, 64, [9]),
+    (3, 10, 6, 32, [4, 9, 2]),  # runs past M: cut off at the last row
+])
+def test_grouped_against_float64_bruteforce(g, m, n, k, sizes):
+    xq, wq, ms, xs, ws = orc.make_grouped_inputs(g, m, n, k, sizes=sizes)
+    got = orc.grouped_dequant_matmul(xq, wq, ms, xs, ws).float().numpy().astype(np.float64)
+    # the brute force applies the same cut at M by construction (rows only run to m - 1)
+    want = _grouped_bruteforce(xq, wq, [int(v) for v in ms], xs, ws)
+    # one bf16 rounding (2^-9 relative) plus fp32 accumulation noise
+    assert np.all(np.abs(got - want) <= np.abs(want) * 2.0 ** -8 + 1e-6)
+
+
+def test_grouped_with_one_group_is_the_plain_product():
+    xq, wq, ms, xs, ws = orc.make_grouped_inputs(1, 24, 10, 96)
+    assert torch.equal(orc.grouped_dequant_matmul(xq, wq, ms, xs, ws), orc.dequant_matmul(xq, wq, xs, ws))
+
+
+def test_grouped_rows_use_their_own_groups_weights_and_scales():
+    # A = ones, B rows of group g all equal to g + 1, K = 16: C = 16 * (g + 1) * a_scale * b_scale
+    g, n, k = 3, 4, 16
+    sizes = [2, 3, 1]
+    m = 8  # two rows more than the sizes cover
+    xq = torch.ones(m, k).to(torch.float8_e4m3fn)
+    wq = torch.cat([torch.full((n, k), float(i + 1)) for i in range(g)]).to(torch.float8_e4m3fn)
+    xs = torch.arange(1, m + 1, dtype=torch.float32)
+    ws = torch.full((g * n,), 0.5)
+    out = orc.grouped_dequant_matmul(xq, wq, torch.tensor(sizes, dtype=torch.int32), xs, ws).float()
+    group_of_row = [0, 0, 1, 1, 1, 2]
+    for r, gi in enumerate(group_of_row):
+        assert torch.all(out[r] == 16.0 * (gi + 1) * (r + 1) * 0.5)
+    assert torch.all(out[6:] == 0)

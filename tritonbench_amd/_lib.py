@@ -49,6 +49,12 @@ SIGNATURES = {
          c_int64, c_int64, c_int64, c_int64, c_int64, c_int64,
          c_void_p, c_size_t, c_int, c_void_p],
     ),
+    "mi355x_fp8_rowwise_grouped_gemm": (
+        c_int,
+        [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
+         c_int64, c_int64, c_int64, c_int64, c_int64, c_int64, c_int64,
+         c_int, c_void_p],
+    ),
     "mi355x_fp8_rowwise_quantize": (
         c_int,
         [c_void_p, c_int, c_void_p, c_void_p, c_int64, c_int64, c_int64, c_int64, c_void_p],

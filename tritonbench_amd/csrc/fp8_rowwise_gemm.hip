@@ -60,6 +60,21 @@ struct GemmParams {
   // partial[split][M][N] and a second kernel adds them up and applies the epilogue
   int splits, steps_per_split;
   float* partial;
+  // grouped form: `groups` consecutive row blocks of A and C, block g of m_sizes[g] rows
+  // (device memory) multiplied with rows [g*N, (g+1)*N) of B and scaled by b_scale[g*N + n]
+  const int32_t* m_sizes;
+  int groups;
+};
+
+// Where a tile sits: rows [m0, m_end) of A and C it may touch, first column, group.
+struct TileLoc {
+  int m0, m_end, n0, group;
+};
+
+// Cursor over the groups for the grouped form. Tiles are numbered group by group; inside a
+// group column-major (consecutive tiles share a B panel). A walker only moves forward.
+struct GroupWalk {
+  int group, tile_begin, tile_end, row_begin, tiles_m;
 };
 
 __device__ __forceinline__ uint16_t f32_to_bf16_rne(float f) {
@@ -186,11 +201,12 @@ constexpr int kEpiPlain = 0, kEpiBias = 1, kEpiPartial = 2;
 constexpr size_t tiled_lds_bytes(int BM, int BN) { return (size_t)(kStagesA * BM + kStagesB * BN) * kStepK; }
 constexpr int tiled_wgs_per_cu(int BM, int BN) { return tiled_lds_bytes(BM, BN) <= 80 * 1024 ? 2 : 1; }
 
-template <int BM, int BN, int WAVES_M, int WAVES_N, bool KTAIL, int EPI>
+template <int BM, int BN, int WAVES_M, int WAVES_N, bool KTAIL, int EPI, bool GROUPED = false>
 __global__ __launch_bounds__(WAVES_M* WAVES_N * 64)
 __attribute__((amdgpu_waves_per_eu(tiled_wgs_per_cu(BM, BN) * WAVES_M * WAVES_N / 4,
                                    tiled_wgs_per_cu(BM, BN) * WAVES_M * WAVES_N / 4)))
 void gemm_tiled_kernel(GemmParams p) {
+  static_assert(!GROUPED || EPI == kEpiPlain, "the grouped form has neither bias nor split-K");
   constexpr bool HAS_BIAS = EPI == kEpiBias;
   constexpr int NW = WAVES_M * WAVES_N;
   constexpr int WTM = BM / WAVES_M;    // wave tile rows (m)
@@ -232,7 +248,17 @@ void gemm_tiled_kernel(GemmParams p) {
 
   // Work items are (split, tile) pairs, split-major: consecutive items are neighbouring
   // tiles of the same K range, so an XCD's chunk of the list still shares operand panels.
-  const int total_tiles = p.tiles_m * p.tiles_n;
+  int total_tiles = p.tiles_m * p.tiles_n;
+  // rows of group g, given the rows before it: never negative, never past row M
+  auto group_rows = [&](int g, int row_begin) { return min(max(p.m_sizes[g], 0), p.M - row_begin); };
+  if (GROUPED) {
+    total_tiles = 0;
+    for (int g = 0, rows = 0; g < p.groups; ++g) {
+      const int mg = group_rows(g, rows);
+      total_tiles += ((mg + BM - 1) / BM) * p.tiles_n;
+      rows += mg;
+    }
+  }
   const TileWalk walk = make_walk(total_tiles * p.splits);
   if (walk.slot >= walk.chunk_len) return;  // uniform over the workgroup
   const int k_full = p.K / kStepK;             // whole 128-byte steps
@@ -246,6 +272,36 @@ void gemm_tiled_kernel(GemmParams p) {
   for (int li = walk.slot; li < walk.chunk_len; li += walk.slots)
     total_steps += split_end(item_split(li)) - split_begin(item_split(li));
 
+  // item -> tile location. Plain form: grouped walk order over the tile grid. Grouped form:
+  // the walker steps through m_sizes until it reaches the group that holds the tile.
+  auto locate = [&](GroupWalk& w, int li) -> TileLoc {
+    const int tile = item_tile(li);
+    if (!GROUPED) {
+      int tm, tn;
+      tile_coords(tile, p.tiles_m, p.tiles_n, p.group_m, tm, tn);
+      return TileLoc{tm * BM, p.M, tn * BN, 0};
+    }
+    while (tile >= w.tile_end && w.group + 1 < p.groups) {
+      w.row_begin += group_rows(w.group, w.row_begin);
+      ++w.group;
+      w.tiles_m = (group_rows(w.group, w.row_begin) + BM - 1) / BM;
+      w.tile_begin = w.tile_end;
+      w.tile_end += w.tiles_m * p.tiles_n;
+    }
+    const int t = tile - w.tile_begin;
+    const int tm = t % max(w.tiles_m, 1), tn = t / max(w.tiles_m, 1);
+    return TileLoc{w.row_begin + tm * BM, w.row_begin + group_rows(w.group, w.row_begin), tn * BN, w.group};
+  };
+  auto first_group = [&]() -> GroupWalk {
+    GroupWalk w = {0, 0, 0, 0, 0};
+    if (GROUPED) {
+      w.tiles_m = (group_rows(0, 0) + BM - 1) / BM;
+      w.tile_end = w.tiles_m * p.tiles_n;
+    }
+    return w;
+  };
+  GroupWalk walk_a = first_group(), walk_b = first_group(), walk_c = first_group();
+
   // ---- load side of the pipeline
   StepCursor ca = {walk.slot, 0, 0, 0}, cb = {walk.slot, 0, 0, 0};
   const uint8_t* l_a = nullptr;
@@ -254,25 +310,23 @@ void gemm_tiled_kernel(GemmParams p) {
   // Rows past the matrix edge are redirected to the last valid row: they are read but never
   // stored, so every load stays in bounds without predication.
   auto setup_a = [&](int li) {
-    int tm, tn;
-    tile_coords(item_tile(li), p.tiles_m, p.tiles_n, p.group_m, tm, tn);
+    const TileLoc loc = locate(walk_a, li);
     ca.kt = split_begin(item_split(li));
     ca.kt_end = split_end(item_split(li));
-    const int m0 = tm * BM;
+    const int m0 = loc.m0;
     l_a = p.a + (size_t)m0 * p.lda;
 #pragma unroll
     for (int i = 0; i < A_GROUPS; ++i) {
       const int grp = wave + NW * i;
-      a_off[i] = (uint32_t)min(grp * 8 + ld_row, p.M - 1 - m0) * (uint32_t)p.lda + ld_chunk_off(grp);
+      a_off[i] = (uint32_t)min(grp * 8 + ld_row, loc.m_end - 1 - m0) * (uint32_t)p.lda + ld_chunk_off(grp);
     }
   };
   auto setup_b = [&](int li) {
-    int tm, tn;
-    tile_coords(item_tile(li), p.tiles_m, p.tiles_n, p.group_m, tm, tn);
+    const TileLoc loc = locate(walk_b, li);
     cb.kt = split_begin(item_split(li));
     cb.kt_end = split_end(item_split(li));
-    const int n0 = tn * BN;
-    l_b = p.b + (size_t)n0 * p.ldb;
+    const int n0 = loc.n0;
+    l_b = p.b + ((size_t)loc.group * p.N + n0) * p.ldb;
 #pragma unroll
     for (int i = 0; i < B_GROUPS; ++i) {
       const int grp = wave + NW * i;
@@ -398,7 +452,9 @@ void gemm_tiled_kernel(GemmParams p) {
   constexpr int LPR = CPR / 2;                  // lanes per row when reading back (2 chunks each)
   constexpr int ROWS_PER_READ = 64 / LPR;
   static_assert(B_GROUPS % 4 == 0 && NT % PASS_J == 0 && (CPR == 8 || CPR == 16), "turn-table geometry");
-  auto epilogue = [&](int m0, int n0, auto aligned_tag, uint8_t* free_b_stage) {
+  auto epilogue = [&](const TileLoc& loc, auto aligned_tag, uint8_t* free_b_stage) {
+    const int m0 = loc.m0, n0 = loc.n0;
+    const float* const b_scale = p.b_scale + (GROUPED ? (size_t)loc.group * p.N : 0);
     constexpr bool ALIGNED = decltype(aligned_tag)::value;  // whole tile inside C, rows 16-byte aligned
     auto row_addr = [&](int r) -> uint8_t* {
       return free_b_stage + (wave + NW * (r / ROWS_PER_GROUP)) * 1024 + (r % ROWS_PER_GROUP) * ROW_BYTES;
@@ -416,12 +472,12 @@ void gemm_tiled_kernel(GemmParams p) {
 
     float sam[MT], sbv[NJP][8], bv[NJP][8];
 #pragma unroll
-    for (int i = 0; i < MT; ++i) sam[i] = p.a_scale[min(m0 + wm * WTM + i * 32 + l32, p.M - 1)];
+    for (int i = 0; i < MT; ++i) sam[i] = p.a_scale[min(m0 + wm * WTM + i * 32 + l32, loc.m_end - 1)];
 #pragma unroll
     for (int jp = 0; jp < NJP; ++jp) {
       const int n = n0 + wn * WTN + jp * PASS_J * 32 + rd_col;
       if (ALIGNED) {
-        const v4f s0 = *(const v4f*)(p.b_scale + n), s1 = *(const v4f*)(p.b_scale + n + 4);
+        const v4f s0 = *(const v4f*)(b_scale + n), s1 = *(const v4f*)(b_scale + n + 4);
 #pragma unroll
         for (int e = 0; e < 4; ++e) sbv[jp][e] = s0[e], sbv[jp][4 + e] = s1[e];
         if (HAS_BIAS) {
@@ -432,7 +488,7 @@ void gemm_tiled_kernel(GemmParams p) {
       } else {
 #pragma unroll
         for (int e = 0; e < 8; ++e) {
-          sbv[jp][e] = p.b_scale[min(n + e, p.N - 1)];
+          sbv[jp][e] = b_scale[min(n + e, p.N - 1)];
           if (HAS_BIAS) bv[jp][e] = bf16_to_f32(p.bias[min(n + e, p.N - 1)]);
         }
       }
@@ -481,7 +537,7 @@ void gemm_tiled_kernel(GemmParams p) {
           uint16_t* dst = p.c + (size_t)m * p.ldc + n;
           if (ALIGNED) {
             *(v4i*)dst = out;
-          } else if (m < p.M) {
+          } else if (m < loc.m_end) {
 #pragma unroll
             for (int e = 0; e < 8; ++e)
               if (n + e < p.N) dst[e] = (uint16_t)((unsigned)out[e / 2] >> (16 * (e & 1)));
@@ -611,18 +667,18 @@ void gemm_tiled_kernel(GemmParams p) {
       step(std::false_type{}, std::false_type{});
     }
     {
-      int tm, tn;
-      tile_coords(item_tile(c_item), p.tiles_m, p.tiles_n, p.group_m, tm, tn);
-      const int m0 = tm * BM, n0 = tn * BN;
+      const TileLoc loc = locate(walk_c, c_item);
       if (EPI == kEpiPartial) {
-        store_partial(m0, n0, c_split);
+        store_partial(loc.m0, loc.n0, c_split);
       } else {
         // sb already names the next step's stage; the one before it held this tile's last step
         uint8_t* free_b = lds + LDS_B0 + ((sb + kStagesB - 1) % kStagesB) * STAGE_B;
-        const bool interior = (m0 + BM <= p.M) && (n0 + BN <= p.N);
-        const uintptr_t c_bits = reinterpret_cast<uintptr_t>(p.c) | (uintptr_t)(p.ldc * 2);
-        if (interior && (c_bits & 15) == 0) epilogue(m0, n0, std::true_type{}, free_b);
-        else epilogue(m0, n0, std::false_type{}, free_b);
+        const bool interior = (loc.m0 + BM <= loc.m_end) && (loc.n0 + BN <= p.N);
+        // b_scale is read 16 bytes at a time on this path: a group's slice must start aligned
+        const uintptr_t bits = reinterpret_cast<uintptr_t>(p.c) | (uintptr_t)(p.ldc * 2) |
+                               (GROUPED ? (uintptr_t)(p.N * 4) : 0);
+        if (interior && (bits & 15) == 0) epilogue(loc, std::true_type{}, free_b);
+        else epilogue(loc, std::false_type{}, free_b);
       }
     }
     read_first_half();  // of the next item's first step (landed before this item's last barrier)
@@ -1153,17 +1209,18 @@ inline TiledPlan plan_from_variant(int64_t M, int64_t N, int64_t K, int variant,
   return plan_tiled(M, N, K, cfg, spl, spl > 0 ? spl : max_splits);
 }
 
-template <int BM, int BN, int WAVES_M, int WAVES_N, bool KTAIL, int EPI>
+template <int BM, int BN, int WAVES_M, int WAVES_N, bool KTAIL, int EPI, bool GROUPED = false>
 int launch_tiled(GemmParams p, hipStream_t stream) {
   constexpr int threads = WAVES_M * WAVES_N * 64;
   constexpr size_t lds_bytes = tiled_lds_bytes(BM, BN);
-  p.tiles_m = (p.M + BM - 1) / BM;
+  // grouped: the group sizes live on the device; every group adds at most one partial tile row
+  p.tiles_m = GROUPED ? p.M / BM + p.groups : (p.M + BM - 1) / BM;
   p.tiles_n = (p.N + BN - 1) / BN;
   p.group_m = 4;
   const long total = (long)p.tiles_m * p.tiles_n * p.splits;
   const long slots = (long)kNumCu * tiled_wgs_per_cu(BM, BN);
   long grid = total < slots ? ((total + kNumXcd - 1) / kNumXcd) * kNumXcd : slots;
-  auto kern = gemm_tiled_kernel<BM, BN, WAVES_M, WAVES_N, KTAIL, EPI>;
+  auto kern = gemm_tiled_kernel<BM, BN, WAVES_M, WAVES_N, KTAIL, EPI, GROUPED>;
   static bool attr_set = false;  // raising the dynamic LDS limit is idempotent; races are harmless
   if (!attr_set) {
     hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize,
@@ -1269,6 +1326,7 @@ int mi355x_fp8_rowwise_gemm(const void* a, const void* b, const float* a_scale, 
   p.lda = lda; p.ldb = ldb; p.ldc = ldc;
   p.tiles_m = p.tiles_n = 0; p.group_m = 1;
   p.splits = 1; p.steps_per_split = k_steps_of(K); p.partial = nullptr;
+  p.m_sizes = nullptr; p.groups = 0;
   hipStream_t s = (hipStream_t)stream;
 
   switch (variant) {
@@ -1306,10 +1364,52 @@ int mi355x_fp8_rowwise_gemm(const void* a, const void* b, const float* a_scale, 
       if (M <= 16) return launch_skinny<SKCFG>(p, s);
       if (M <= 32) return launch_skinny<2, 1, 2, 8>(p, s);
       if (M <= 48) return launch_skinny<3, 1, 2, 8>(p, s);
-      return launch_skinny<4, 1, 2, 8>(p, s);
+      return launch_skinny<4, 2, 2, 8>(p, s);  // 32 rows of B per workgroup: A passes L1 half as often
     default:
       return fail(MI355X_FP8_EINVAL, "unknown variant %d", variant);
   }
+}
+
+int mi355x_fp8_rowwise_grouped_gemm(const void* a, const void* b, const float* a_scale, const float* b_scale,
+                                    const int32_t* m_sizes, void* c, int64_t G, int64_t M, int64_t N,
+                                    int64_t K, int64_t lda, int64_t ldb, int64_t ldc, int tile_config,
+                                    void* stream) {
+  int st = check_shape(M, N, K);
+  if (st != MI355X_FP8_OK) return st;
+  if (G < 1 || G > 65536) return fail(MI355X_FP8_EINVAL, "G must be in 1..65536 (got %lld)", (long long)G);
+  if (G * N > INT32_MAX) return fail(MI355X_FP8_ENOTSUP, "G*N exceeds 2^31-1");
+  if (!a || !b || !a_scale || !b_scale || !m_sizes || !c) return fail(MI355X_FP8_EINVAL, "null operand pointer");
+  if (lda < K || ldb < K || ldc < N) return fail(MI355X_FP8_EINVAL, "leading dimension smaller than the row length");
+  if (lda % 16 || ldb % 16) return fail(MI355X_FP8_ENOTSUP, "lda and ldb must be multiples of 16");
+  if ((reinterpret_cast<uintptr_t>(a) & 15) || (reinterpret_cast<uintptr_t>(b) & 15))
+    return fail(MI355X_FP8_ENOTSUP, "a and b must be 16-byte aligned");
+  if ((reinterpret_cast<uintptr_t>(a_scale) & 3) || (reinterpret_cast<uintptr_t>(b_scale) & 15) ||
+      (reinterpret_cast<uintptr_t>(c) & 1) || (reinterpret_cast<uintptr_t>(m_sizes) & 3))
+    return fail(MI355X_FP8_EINVAL, "misaligned scale, size or output pointer (b_scale needs 16 bytes)");
+  if (lda * 256 > (int64_t)UINT32_MAX || ldb * 256 > (int64_t)UINT32_MAX)
+    return fail(MI355X_FP8_ENOTSUP, "leading dimension too large");
+  if (tile_config < -1 || tile_config >= kNumTileConfigs)
+    return fail(MI355X_FP8_EINVAL, "unknown tile configuration %d", tile_config);
+
+  GemmParams p;
+  p.a = (const uint8_t*)a; p.b = (const uint8_t*)b;
+  p.a_scale = a_scale; p.b_scale = b_scale;
+  p.bias = nullptr; p.c = (uint16_t*)c;
+  p.M = (int)M; p.N = (int)N; p.K = (int)K;
+  p.lda = lda; p.ldb = ldb; p.ldc = ldc;
+  p.tiles_m = p.tiles_n = 0; p.group_m = 1;
+  p.splits = 1; p.steps_per_split = k_steps_of(K); p.partial = nullptr;
+  p.m_sizes = m_sizes; p.groups = (int)G;
+  hipStream_t s = (hipStream_t)stream;
+  // Large tiles when an average group fills most of one, small tiles otherwise (the group
+  // sizes themselves are on the device; M / G is what the host knows).
+  if (tile_config < 0) tile_config = (M / G >= 192 && N >= 256) ? 0 : 1;
+  const bool ktail = K % kStepK;
+  if (tile_config == 0)
+    return ktail ? launch_tiled<256, 256, 2, 2, true, kEpiPlain, true>(p, s)
+                 : launch_tiled<256, 256, 2, 2, false, kEpiPlain, true>(p, s);
+  return ktail ? launch_tiled<128, 128, 2, 2, true, kEpiPlain, true>(p, s)
+               : launch_tiled<128, 128, 2, 2, false, kEpiPlain, true>(p, s);
 }
 
 int mi355x_fp8_rowwise_quantize(const void* x, int src_type, void* xq, float* inv_scale, int64_t R,

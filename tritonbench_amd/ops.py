@@ -101,6 +101,60 @@ def fp8_gemm_rowwise(
     return out
 
 
+def fp8_gemm_rowwise_grouped(
+    group_a: torch.Tensor,
+    group_b: torch.Tensor,
+    m_sizes: torch.Tensor,
+    a_scale: torch.Tensor,
+    b_scale: torch.Tensor,
+    out: Optional[torch.Tensor] = None,
+    tile_config: int = -1,
+) -> torch.Tensor:
+    """Grouped row-wise FP8 GEMM: bf16 [M,N], rows of group g = group_a rows of that group times
+    group_b[g*N:(g+1)*N].T, scaled row- and column-wise.
+
+    Same operands as the callables of
+    tritonbench/operators/fp8_gemm_rowwise_grouped/operator.py:400-455: group_a [M,K] and
+    group_b [G*N,K] float8_e4m3fn, m_sizes int32 [G] ON THE DEVICE (never read by the host),
+    a_scale [M] and b_scale [G*N] float32. Rows past sum(m_sizes) keep what `out` held
+    (zeros when this call allocates it). Only enqueues work on the current stream.
+    """
+    lib = _lib.load()
+    for t, name in ((group_a, "group_a"), (group_b, "group_b"), (m_sizes, "m_sizes"), (a_scale, "a_scale"),
+                    (b_scale, "b_scale")):
+        _require_gpu(t, name)
+    if group_a.dtype != FP8_DTYPE or group_b.dtype != FP8_DTYPE:
+        raise TypeError(f"group_a and group_b must be {FP8_DTYPE}")
+    if group_a.dim() != 2 or group_b.dim() != 2 or group_a.shape[1] != group_b.shape[1]:
+        raise ValueError("expected group_a [M,K] and group_b [G*N,K]")
+    if m_sizes.dtype != torch.int32 or m_sizes.dim() != 1 or not m_sizes.is_contiguous() or m_sizes.numel() < 1:
+        raise ValueError("m_sizes must be a contiguous int32 vector with one entry per group")
+    g = m_sizes.numel()
+    m, k = group_a.shape
+    if group_b.shape[0] % g:
+        raise ValueError(f"group_b has {group_b.shape[0]} rows, not a multiple of the {g} groups")
+    n = group_b.shape[0] // g
+    if a_scale.dtype != torch.float32 or b_scale.dtype != torch.float32:
+        raise TypeError("a_scale and b_scale must be float32")
+    if a_scale.numel() != m or b_scale.numel() != g * n or not a_scale.is_contiguous() or not b_scale.is_contiguous():
+        raise ValueError("a_scale must have M entries and b_scale G*N entries, both contiguous")
+    if group_a.stride(1) != 1 or group_b.stride(1) != 1:
+        raise ValueError("group_a and group_b must be K-contiguous")
+    if out is None:
+        out = torch.zeros((m, n), dtype=torch.bfloat16, device=group_a.device)
+    else:
+        _require_gpu(out, "out")
+        if out.dtype != torch.bfloat16 or tuple(out.shape) != (m, n) or out.stride(1) != 1:
+            raise ValueError("out must be bfloat16 [M,N] with unit column stride")
+    st = lib.mi355x_fp8_rowwise_grouped_gemm(
+        group_a.data_ptr(), group_b.data_ptr(), a_scale.data_ptr(), b_scale.data_ptr(), m_sizes.data_ptr(),
+        out.data_ptr(), g, m, n, k, group_a.stride(0), group_b.stride(0), out.stride(0), tile_config,
+        _stream_ptr(),
+    )
+    _lib.check(st, "mi355x_fp8_rowwise_grouped_gemm")
+    return out
+
+
 def fp8_row_quantize(x: torch.Tensor) -> Tuple[torch.Tensor, torch.Tensor]:
     """Row-wise e4m3fn quantisation on the GPU; returns (xq, inverse scale) like
     fp8_row_quantize in tritonbench/operators/fp8_gemm_rowwise/operator.py:136-145."""
