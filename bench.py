@@ -127,6 +127,37 @@ def time_quantiser(r, k, dtype, dev, steps=60, copies=3):
     return dict(us=ms * 1e3, gbps=nbytes / ms / 1e6, bound="hbm", frac=nbytes / ms / 1e6 / PEAK_HBM_GBPS)
 
 
+def time_grouped(g, m, n, k, dev, steps=40, copies=2):
+    """Grouped form (equal groups, as the reference's input generator makes them):
+    flops = 2*M*N*K, bytes = M*K + G*N*K + 2*M*N."""
+    from tritonbench_amd import ops
+
+    gen = torch.Generator(device=dev)
+    gen.manual_seed(SEED + g + m + n + k)
+    sets = []
+    for _ in range(copies):
+        xq, xs = ops.fp8_row_quantize(torch.randn((m, k), generator=gen, device=dev, dtype=torch.float32))
+        wq, ws = ops.fp8_row_quantize(torch.randn((g * n, k), generator=gen, device=dev, dtype=torch.float32))
+        sets.append((xq, wq, xs, ws, torch.zeros((m, n), dtype=torch.bfloat16, device=dev)))
+    sizes = torch.tensor([m // g] * g, dtype=torch.int32, device=dev)
+    for i in range(5):
+        xq, wq, xs, ws, out = sets[i % copies]
+        ops.fp8_gemm_rowwise_grouped(xq, wq, sizes, xs, ws, out=out)
+    torch.cuda.synchronize()
+    stream = torch.cuda.current_stream()
+    start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    start.record(stream)
+    for i in range(steps):
+        xq, wq, xs, ws, out = sets[i % copies]
+        ops.fp8_gemm_rowwise_grouped(xq, wq, sizes, xs, ws, out=out)
+    end.record(stream)
+    torch.cuda.synchronize()
+    ms = start.elapsed_time(end) / steps
+    flops, nbytes = 2 * m * n * k, m * k + g * n * k + 2 * m * n
+    return dict(us=ms * 1e3, tflops=flops / ms / 1e9, gbps=nbytes / ms / 1e6, bound="mfma",
+                frac=flops / ms / 1e9 / PEAK_FP8_TFLOPS)
+
+
 def figures(m, n, k, bias, ms):
     flops = 2 * m * n * k + (2 * m * n if bias else 0)
     nbytes = m * k + n * k + 2 * m * n
@@ -242,6 +273,8 @@ def main():
             del rs
         make_device_inputs(m, n, k, 1.0, False, dev, copies=0)  # workspace of the headline plan again
         configs["c2_square_8192_graph"] = figures(m, n, k, False, time_steps_graph(sets, 20, 2))
+        configs["grouped_g4_8192x4096x4096"] = time_grouped(4, 8192, 4096, 4096, dev)
+        configs["grouped_g16_8192x8192x8192"] = time_grouped(16, 8192, 8192, 8192, dev, steps=20)
         configs["quantise_f32_8192x8192"] = time_quantiser(8192, 8192, torch.float32, dev)
         configs["quantise_bf16_8192x8192"] = time_quantiser(8192, 8192, torch.bfloat16, dev)
         configs["quantise_bf16_57344x8192"] = time_quantiser(57344, 8192, torch.bfloat16, dev, steps=20, copies=2)

@@ -3,7 +3,7 @@
 The tritonbench checkout holds no golden vectors or known-answer tests for
 fp8_gemm_rowwise (the operator is skipped by its CI), so the vectors are produced here:
 seeded inputs, quantised by oracle.fp8_rowwise.fp8_row_quantize, outputs from
-oracle.fp8_rowwise.dequant_matmul. Each .npz holds raw arrays only (uint8 e4m3fn codes,
+oracle.fp8_rowwise.dequant_matmul (grouped_dequant_matmul for the grouped cases). Each .npz holds raw arrays only (uint8 e4m3fn codes,
 float32 scales, uint16 bf16 bit patterns); load with allow_pickle=False.
 
     python tests/golden/make_golden.py
@@ -31,6 +31,13 @@ CASES = [
 ]
 
 
+GROUPED_CASES = [
+    # name, g, m, n, k, sizes
+    ("grouped_g3_300x72x144", 3, 300, 72, 144, [130, 0, 150]),  # an empty group; 20 rows owned by no group
+    ("grouped_g2_64x33x272", 2, 64, 33, 272, None),              # equal split, N not a multiple of 4
+]
+
+
 def main():
     manifest = {"generator": "tests/golden/make_golden.py", "seed": orc.MAIN_RANDOM_SEED, "cases": []}
     for name, m, n, k, sigma, bias in CASES:
@@ -49,9 +56,25 @@ def main():
         np.savez_compressed(os.path.join(HERE, fname), **arrays)
         digest = hashlib.sha256(b"".join(np.ascontiguousarray(v).tobytes() for _, v in sorted(arrays.items()))).hexdigest()
         manifest["cases"].append(dict(name=name, file=fname, m=m, n=n, k=k, sigma=sigma, bias=bias, sha256=digest))
+    manifest["grouped_cases"] = []
+    for name, g, m, n, k, sizes in GROUPED_CASES:
+        xq, wq, ms, xs, ws = orc.make_grouped_inputs(g, m, n, k, sizes=sizes)
+        out = orc.grouped_dequant_matmul(xq, wq, ms, xs, ws)
+        arrays = dict(
+            a=xq.view(torch.uint8).numpy(),
+            b=wq.view(torch.uint8).numpy(),
+            m_sizes=ms.numpy(),
+            a_scale=xs.numpy(),
+            b_scale=ws.numpy(),
+            c=out.view(torch.int16).numpy().view(np.uint16),
+        )
+        fname = name + ".npz"
+        np.savez_compressed(os.path.join(HERE, fname), **arrays)
+        digest = hashlib.sha256(b"".join(np.ascontiguousarray(v).tobytes() for _, v in sorted(arrays.items()))).hexdigest()
+        manifest["grouped_cases"].append(dict(name=name, file=fname, g=g, m=m, n=n, k=k, sha256=digest))
     with open(os.path.join(HERE, "manifest.json"), "w") as f:
         json.dump(manifest, f, indent=1)
-    print(f"wrote {len(CASES)} cases")
+    print(f"wrote {len(CASES)} + {len(GROUPED_CASES)} cases")
 
 
 if __name__ == "__main__":

@@ -48,6 +48,25 @@ def _check(out, want, operands=None):
         start = end
 
 
+def test_grouped_golden_fixtures(gpu_device):
+    import json
+    import os
+
+    golden = os.path.join(os.path.dirname(__file__), "golden")
+    with open(os.path.join(golden, "manifest.json")) as f:
+        manifest = json.load(f)
+    for case in manifest["grouped_cases"]:
+        z = np.load(os.path.join(golden, case["file"]), allow_pickle=False)
+        xq = torch.from_numpy(z["a"]).view(torch.float8_e4m3fn)
+        wq = torch.from_numpy(z["b"]).view(torch.float8_e4m3fn)
+        ms, xs, ws = torch.from_numpy(z["m_sizes"]), torch.from_numpy(z["a_scale"]), torch.from_numpy(z["b_scale"])
+        want = torch.from_numpy(z["c"].view(np.int16)).view(torch.bfloat16)
+        for cfg in [-1] + list(range(_lib.NUM_TILE_CONFIGS)):
+            print(f"golden {case['name']} tile_config {cfg}", flush=True)
+            out = _run(gpu_device, xq, wq, ms, xs, ws, cfg)  # allocated by the call: unowned rows are zero
+            _check(out, want, (xq, wq, ms, xs, ws))
+
+
 CASES = [
     # g, m, n, k, sizes (None = equal split as the reference's input generator makes them)
     (2, 1024, 1024, 1024, None),

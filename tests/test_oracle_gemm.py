@@ -170,7 +170,7 @@ def _grouped_bruteforce(xq, wq, sizes, xs, ws):
     a = e4m3.decode(xq.view(torch.uint8).numpy()).astype(np.float64)
     b = e4m3.decode(wq.view(torch.uint8).numpy()).astype(np.float64)
     m, n = a.shape[0], b.shape[0] // len(sizes)
-    out = np.zeros((m, n))
+    out, mag = np.zeros((m, n)), np.zeros((m, n))
     bounds = np.cumsum([0] + [max(int(s), 0) for s in sizes])
     for r in range(m):
         g = int(np.searchsorted(bounds, r, side="right")) - 1
@@ -178,7 +178,9 @@ def _grouped_bruteforce(xq, wq, sizes, xs, ws):
             continue  # past the last group: stays zero
         for c in range(n):
             out[r, c] = np.dot(a[r], b[g * n + c]) * float(xs[r]) * float(ws[g * n + c])
-    return out
+            mag[r, c] = np.dot(np.abs(a[r]), np.abs(b[g * n + c])) * float(xs[r]) * float(ws[g * n + c])
+    # second value: what fp32 accumulation in any order may add to the error
+    return out, mag * a.shape[1] * 2.0 ** -24
 
 
 @pytest.mark.parametrize("g,m,n,k,sizes", [
@@ -189,9 +191,9 @@ def test_grouped_against_float64_bruteforce(g, m, n, k, sizes):
     xq, wq, ms, xs, ws = orc.make_grouped_inputs(g, m, n, k, sizes=sizes)
     got = orc.grouped_dequant_matmul(xq, wq, ms, xs, ws).float().numpy().astype(np.float64)
     # the brute force applies the same cut at M by construction (rows only run to m - 1)
-    want = _grouped_bruteforce(xq, wq, [int(v) for v in ms], xs, ws)
+    want, slack = _grouped_bruteforce(xq, wq, [int(v) for v in ms], xs, ws)
     # one bf16 rounding (2^-9 relative) plus fp32 accumulation noise
-    assert np.all(np.abs(got - want) <= np.abs(want) * 2.0 ** -8 + 1e-6)
+    assert np.all(np.abs(got - want) <= np.abs(want) * 2.0 ** -8 + slack)
 
 
 def test_grouped_with_one_group_is_the_plain_product():
@@ -213,3 +215,22 @@ def test_grouped_rows_use_their_own_groups_weights_and_scales():
     for r, gi in enumerate(group_of_row):
         assert torch.all(out[r] == 16.0 * (gi + 1) * (r + 1) * 0.5)
     assert torch.all(out[6:] == 0)
+
+
+def test_grouped_golden_fixtures_match_oracle_and_bruteforce():
+    with open(os.path.join(GOLDEN, "manifest.json")) as f:
+        manifest = json.load(f)
+    assert manifest["grouped_cases"], "no grouped golden cases"
+    for case in manifest["grouped_cases"]:
+        z = np.load(os.path.join(GOLDEN, case["file"]), allow_pickle=False)
+        g, m, n, k = case["g"], case["m"], case["n"], case["k"]
+        assert z["a"].shape == (m, k) and z["b"].shape == (g * n, k) and z["c"].shape == (m, n)
+        assert z["m_sizes"].dtype == np.int32 and z["m_sizes"].shape == (g,)
+        xq = torch.from_numpy(z["a"]).view(torch.float8_e4m3fn)
+        wq = torch.from_numpy(z["b"]).view(torch.float8_e4m3fn)
+        xs, ws = torch.from_numpy(z["a_scale"]), torch.from_numpy(z["b_scale"])
+        out = orc.grouped_dequant_matmul(xq, wq, torch.from_numpy(z["m_sizes"]), xs, ws)
+        assert np.mean(_bits(out) == z["c"]) > 0.99, case["name"]
+        want = orc.bf16_bits_to_f32(z["c"]).astype(np.float64)
+        exact, slack = _grouped_bruteforce(xq, wq, z["m_sizes"].tolist(), xs, ws)
+        assert np.all(np.abs(want - exact) <= np.abs(exact) * 2.0 ** -8 + slack), case["name"]

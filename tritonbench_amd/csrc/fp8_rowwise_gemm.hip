@@ -1401,9 +1401,10 @@ int mi355x_fp8_rowwise_grouped_gemm(const void* a, const void* b, const float* a
   p.splits = 1; p.steps_per_split = k_steps_of(K); p.partial = nullptr;
   p.m_sizes = m_sizes; p.groups = (int)G;
   hipStream_t s = (hipStream_t)stream;
-  // Large tiles when an average group fills most of one, small tiles otherwise (the group
-  // sizes themselves are on the device; M / G is what the host knows).
-  if (tile_config < 0) tile_config = (M / G >= 192 && N >= 256) ? 0 : 1;
+  // Large tiles when an average group fills most of one and there are enough of them for every
+  // CU, small tiles otherwise (the group sizes themselves are on the device; M / G is what the
+  // host knows).
+  if (tile_config < 0) tile_config = (M / G >= 192 && (M / 256) * (N / 256) >= 192) ? 0 : 1;
   const bool ktail = K % kStepK;
   if (tile_config == 0)
     return ktail ? launch_tiled<256, 256, 2, 2, true, kEpiPlain, true>(p, s)
