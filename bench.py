@@ -207,6 +207,8 @@ def main():
     ap.add_argument("--all-configs", action="store_true", help="also time every Llama-3-70B projection shape")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-extra", action="store_true", help="headline workload only")
+    ap.add_argument("--profile-kernel", choices=["skinny", "quantise", "grouped"],
+                    help="run only that kernel's workload a few times (for rocprofv3 counter passes) and print its figures")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py measures one GPU: this hot path is a single-device kernel and nothing here "
@@ -220,6 +222,18 @@ def main():
     _lib.load()
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
+
+    if args.profile_kernel:
+        if args.profile_kernel == "skinny":
+            ps = make_device_inputs(16, 8192, 8192, 1.0, False, dev, copies=10)
+            fig = figures(16, 8192, 8192, False, time_steps(ps, 40, 10))
+        elif args.profile_kernel == "quantise":
+            fig = {"f32": time_quantiser(8192, 8192, torch.float32, dev, steps=20),
+                   "bf16": time_quantiser(8192, 8192, torch.bfloat16, dev, steps=20)}
+        else:
+            fig = time_grouped(4, 8192, 4096, 4096, dev, steps=20)
+        print(json.dumps({"profile_kernel": args.profile_kernel, "figures": fig}))
+        return
 
     m = n = k = 8192
     sets = make_device_inputs(m, n, k, 1.0, False, dev, copies=1)

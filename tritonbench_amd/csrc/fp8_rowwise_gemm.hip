@@ -1209,6 +1209,20 @@ inline TiledPlan plan_from_variant(int64_t M, int64_t N, int64_t K, int variant,
   return plan_tiled(M, N, K, cfg, spl, spl > 0 ? spl : max_splits);
 }
 
+// Raises a kernel's dynamic-LDS limit once per device (the attribute belongs to the device's
+// copy of the code object). Idempotent, so a race between threads is harmless.
+constexpr int kMaxDevices = 64;
+int raise_lds_limit(const void* kernel, size_t lds_bytes, bool (&done)[kMaxDevices]) {
+  int dev = 0;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) return fail(MI355X_FP8_ELAUNCH, "hipGetDevice: %s", hipGetErrorString(e));
+  if (dev >= 0 && dev < kMaxDevices && done[dev]) return MI355X_FP8_OK;
+  e = hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
+  if (e != hipSuccess) return fail(MI355X_FP8_ELAUNCH, "hipFuncSetAttribute: %s", hipGetErrorString(e));
+  if (dev >= 0 && dev < kMaxDevices) done[dev] = true;
+  return MI355X_FP8_OK;
+}
+
 template <int BM, int BN, int WAVES_M, int WAVES_N, bool KTAIL, int EPI, bool GROUPED = false>
 int launch_tiled(GemmParams p, hipStream_t stream) {
   constexpr int threads = WAVES_M * WAVES_N * 64;
@@ -1221,13 +1235,8 @@ int launch_tiled(GemmParams p, hipStream_t stream) {
   const long slots = (long)kNumCu * tiled_wgs_per_cu(BM, BN);
   long grid = total < slots ? ((total + kNumXcd - 1) / kNumXcd) * kNumXcd : slots;
   auto kern = gemm_tiled_kernel<BM, BN, WAVES_M, WAVES_N, KTAIL, EPI, GROUPED>;
-  static bool attr_set = false;  // raising the dynamic LDS limit is idempotent; races are harmless
-  if (!attr_set) {
-    hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize,
-                                       (int)lds_bytes);
-    if (e != hipSuccess) return fail(MI355X_FP8_ELAUNCH, "hipFuncSetAttribute: %s", hipGetErrorString(e));
-    attr_set = true;
-  }
+  static bool attr_done[kMaxDevices] = {};
+  if (const int st = raise_lds_limit((const void*)kern, lds_bytes, attr_done)) return st;
   hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(threads), lds_bytes, stream, p);
   hipError_t e = hipGetLastError();
   if (e != hipSuccess) return fail(MI355X_FP8_ELAUNCH, "tiled kernel launch: %s", hipGetErrorString(e));
@@ -1258,12 +1267,8 @@ int launch_skinny(const GemmParams& p, hipStream_t stream) {
   constexpr size_t lds_bytes = (size_t)KW * (NTW + MT) * 16 * kStepK;
   static_assert(lds_bytes <= 160 * 1024, "transpose buffers must fit the 160 KB LDS");
   auto kern = gemm_skinny_kernel<MT, NTW, DEPTH, KW>;
-  static bool attr_set = false;
-  if (!attr_set) {
-    hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
-    if (e != hipSuccess) return fail(MI355X_FP8_ELAUNCH, "hipFuncSetAttribute: %s", hipGetErrorString(e));
-    attr_set = true;
-  }
+  static bool attr_done[kMaxDevices] = {};
+  if (const int st = raise_lds_limit((const void*)kern, lds_bytes, attr_done)) return st;
   const unsigned grid = (unsigned)((p.N + 16 * NTW - 1) / (16 * NTW));
   hipLaunchKernelGGL(kern, dim3(grid), dim3(KW * 64), lds_bytes, stream, p);
   hipError_t e = hipGetLastError();
