@@ -134,6 +134,26 @@ int mi355x_fp8_rowwise_grouped_gemm(const void* a, const void* b,
                                     int tile_config, void* stream);
 
 /*
+ * Block-scaled form: one scale per 128x128 block of A and of B,
+ *
+ *   C[m, n] = bf16( sum_kb (sum_{k in block kb} A[m,k] * B[n,k]) * a_scale[m/128][kb] * b_scale[n/128][kb] )
+ *
+ * Replaces the timed callables of tritonbench/operators/fp8_gemm_blockwise/operator.py:139-145
+ * (matmul_fp8_block(xq, wq, x_scale, w_scale), f8f8bf16_blockwise(...)); the scale layout is
+ * the one fp8_block_quantize returns there (:86-118).
+ *
+ *   a        e4m3fn [M, K]                        b        e4m3fn [N, K]
+ *   a_scale  f32 [ceil(M/128)][ceil(K/128)]       b_scale  f32 [ceil(N/128)][ceil(K/128)]
+ *   c        bf16 [M, N]
+ *
+ * Requirements as for mi355x_fp8_rowwise_gemm, and K <= 32768.
+ */
+int mi355x_fp8_blockwise_gemm(const void* a, const void* b,
+                              const float* a_scale, const float* b_scale, void* c,
+                              int64_t M, int64_t N, int64_t K,
+                              int64_t lda, int64_t ldb, int64_t ldc, void* stream);
+
+/*
  * Row-wise e4m3fn quantiser, replacing fp8_row_quantize (operator.py:136-145):
  *   amax[r]      = max_k |x[r,k]|
  *   scale[r]     = fl(fl(1 / max(amax[r], 1e-12)) * 448)   (how PyTorch evaluates 448 / tensor)

@@ -176,6 +176,43 @@ def make_inputs(m: int, n: int, k: int, sigma: float = 1.0, bias: bool = False):
 
 
 # The five workload families the parity and bench code iterate over.
+def fp8_block_quantize(x: torch.Tensor, block_m: int = 128, block_k: int = 128) -> Tuple[torch.Tensor, torch.Tensor]:
+    """One scale per block_m x block_k block. Follows fp8_block_quantize,
+    tritonbench/operators/fp8_gemm_blockwise/operator.py:86-118: zero-pad to whole blocks,
+    block_max = amax |x| per block clamped at 1e-12, scale = 448 / block_max (in fp32), a scale
+    of inf becomes 1, xq = (x * scale).to(e4m3fn) (no clamp: |x * scale| <= 448 up to rounding),
+    returns (xq, 1 / scale) with the scale grid [ceil(M/block_m), ceil(K/block_k)]."""
+    m, k = x.shape
+    gm, gk = -(-m // block_m), -(-k // block_k)
+    padded = torch.zeros(gm * block_m, gk * block_k, dtype=x.dtype)
+    padded[:m, :k] = x
+    block_max = padded.abs().reshape(gm, block_m, gk, block_k).amax(dim=(1, 3))
+    block_max = torch.clamp(block_max, min=EPS)
+    scale = E4M3_MAX_POS / block_max.to(torch.float32)
+    scale[scale == float("inf")] = 1.0
+    xq = (padded * scale.repeat_interleave(block_m, dim=0).repeat_interleave(block_k, dim=1))[:m, :k]
+    return xq.to(FP8_DTYPE), 1 / scale
+
+
+def blockwise_dequant_matmul(xq, wq, x_scale, w_scale, block: int = 128) -> torch.Tensor:
+    """Block-scaled product on the CPU: every element is widened to fp32 and multiplied by its
+    block's scale, then one fp32 matmul and one bf16 rounding. Mathematically the sum over K
+    blocks of (xq_blk @ wq_blk.T) * x_scale[m // 128, kb] * w_scale[n // 128, kb] that the
+    callables at tritonbench/operators/fp8_gemm_blockwise/operator.py:139-145 compute."""
+    m, k = xq.shape
+    n = wq.shape[0]
+    xs = x_scale.repeat_interleave(block, dim=0).repeat_interleave(block, dim=1)[:m, :k]
+    ws = w_scale.repeat_interleave(block, dim=0).repeat_interleave(block, dim=1)[:n, :k]
+    return ((xq.to(torch.float32) * xs) @ (wq.to(torch.float32) * ws).t()).to(torch.bfloat16)
+
+
+def make_blockwise_inputs(m, n, k, sigma=1.0, seed_tag=0):
+    """Seeded operands of the block-scaled form, quantised per 128x128 block."""
+    xq, xs = fp8_block_quantize(randn_f32(m, k, sigma, seed=MAIN_RANDOM_SEED + 13 * m + k + seed_tag))
+    wq, ws = fp8_block_quantize(randn_f32(n, k, sigma, seed=MAIN_RANDOM_SEED + 29 * n + k + seed_tag))
+    return xq, wq, xs, ws
+
+
 def grouped_dequant_matmul(xq, wq, m_sizes, x_scale, w_scale):
     """Grouped form on the CPU: rows of group g (m_sizes[g] consecutive rows, in order) times
     wq[g*N:(g+1)*N].T with both scales, fp32 dequantise + matmul, one bf16 rounding; rows past

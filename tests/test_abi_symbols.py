@@ -12,7 +12,7 @@ HEADER = os.path.join(ROOT, "include", "mi355x_fp8_rowwise.h")
 def _declared_functions():
     text = open(HEADER).read()
     text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
-    return sorted(set(re.findall(r"\b(mi355x_fp8_rowwise_\w+)\s*\(", text)))
+    return sorted(set(re.findall(r"\b(mi355x_fp8_[a-z]\w+)\s*\(", text)))
 
 
 def test_header_declares_the_expected_entry_points():

@@ -55,6 +55,11 @@ SIGNATURES = {
          c_int64, c_int64, c_int64, c_int64, c_int64, c_int64, c_int64,
          c_int, c_void_p],
     ),
+    "mi355x_fp8_blockwise_gemm": (
+        c_int,
+        [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
+         c_int64, c_int64, c_int64, c_int64, c_int64, c_int64, c_void_p],
+    ),
     "mi355x_fp8_rowwise_quantize": (
         c_int,
         [c_void_p, c_int, c_void_p, c_void_p, c_int64, c_int64, c_int64, c_int64, c_void_p],

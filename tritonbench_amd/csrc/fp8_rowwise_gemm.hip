@@ -199,14 +199,26 @@ struct StepCursor {
 constexpr int kEpiPlain = 0, kEpiBias = 1, kEpiPartial = 2;
 
 constexpr size_t tiled_lds_bytes(int BM, int BN) { return (size_t)(kStagesA * BM + kStagesB * BN) * kStepK; }
-constexpr int tiled_wgs_per_cu(int BM, int BN) { return tiled_lds_bytes(BM, BN) <= 80 * 1024 ? 2 : 1; }
+// (the block-scaled form keeps a second accumulator set and needs the whole register file)
+constexpr int tiled_wgs_per_cu(int BM, int BN, bool blockscale = false) {
+  return !blockscale && tiled_lds_bytes(BM, BN) <= 80 * 1024 ? 2 : 1;
+}
 
-template <int BM, int BN, int WAVES_M, int WAVES_N, bool KTAIL, int EPI, bool GROUPED = false>
+//
+// BLOCKSCALE turns the kernel into the 128x128x128 block-scaled GEMM: a_scale is then
+// [ceil(M/128)][ceil(K/128)], b_scale [ceil(N/128)][ceil(K/128)], and every K step's product
+// is multiplied by a_scale[mb][kb] * b_scale[nb][kb] before it is added up. With 128x128 tiles
+// and 128-byte steps that factor is one number per workgroup and step: the MFMAs of a step
+// go to a second accumulator set, which is folded into the first (acc += s * tmp) behind
+// the next step's MFMAs.
+template <int BM, int BN, int WAVES_M, int WAVES_N, bool KTAIL, int EPI, bool GROUPED = false, bool BLOCKSCALE = false>
 __global__ __launch_bounds__(WAVES_M* WAVES_N * 64)
-__attribute__((amdgpu_waves_per_eu(tiled_wgs_per_cu(BM, BN) * WAVES_M * WAVES_N / 4,
-                                   tiled_wgs_per_cu(BM, BN) * WAVES_M * WAVES_N / 4)))
+__attribute__((amdgpu_waves_per_eu(tiled_wgs_per_cu(BM, BN, BLOCKSCALE) * WAVES_M * WAVES_N / 4,
+                                   tiled_wgs_per_cu(BM, BN, BLOCKSCALE) * WAVES_M * WAVES_N / 4)))
 void gemm_tiled_kernel(GemmParams p) {
   static_assert(!GROUPED || EPI == kEpiPlain, "the grouped form has neither bias nor split-K");
+  static_assert(!BLOCKSCALE || (BM == 128 && BN == 128 && EPI == kEpiPlain && !GROUPED),
+                "block scales are per 128x128 tile: one tile, one scale per step");
   constexpr bool HAS_BIAS = EPI == kEpiBias;
   constexpr int NW = WAVES_M * WAVES_N;
   constexpr int WTM = BM / WAVES_M;    // wave tile rows (m)
@@ -392,13 +404,47 @@ void gemm_tiled_kernel(GemmParams p) {
   };
 
   v16f acc[MT][NT];  // defined by the first step of every work item
+  // BLOCKSCALE only: the running step's unscaled product, the factor it is waiting for, the
+  // K step the compute side is at, and the lane's share of the item's factors
+  // (sc[r] belongs to step 64*r + lane).
+  v16f tmp[BLOCKSCALE ? MT : 1][BLOCKSCALE ? NT : 1];
+  float s_pend = 0.0f;
+  int kt_c = 0;
+  constexpr int SC_REGS = 4;  // 256 steps = K up to 32768
+  float sc[SC_REGS] = {0.f, 0.f, 0.f, 0.f};
+  auto load_block_scales = [&](const TileLoc& loc) {
+    const float* sa = p.a_scale + (size_t)(loc.m0 / 128) * k_steps;
+    const float* sb = p.b_scale + (size_t)(loc.n0 / 128) * k_steps;
+#pragma unroll
+    for (int r = 0; r < SC_REGS; ++r) {
+      const int kb = min(r * 64 + lane, k_steps - 1);
+      sc[r] = sa[kb] * sb[kb];
+    }
+  };
+  auto step_scale = [&](int kt) -> float {
+    const int r = kt >> 6;
+    const float v = r == 0 ? sc[0] : r == 1 ? sc[1] : r == 2 ? sc[2] : sc[3];
+    return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), kt & 63));
+  };
+  // folds block t of the waiting product into the accumulators (or starts them from zero)
+  auto fold_block = [&](int t, bool start) {
+    const int i = t / NT, j = t % NT;
+    auto& tm = tmp[BLOCKSCALE ? i : 0][BLOCKSCALE ? j : 0];
+#pragma unroll
+    for (int v = 0; v < 16; ++v) acc[i][j][v] = start ? 0.0f : __builtin_fmaf(s_pend, tm[v], acc[i][j][v]);
+  };
 
   // t-th MFMA of a half step (t = i*NT + j) on fragment set (fa, fb)
   // (fresh: the block's first MFMA of a tile starts from zero instead of the old contents)
   auto mfma_one = [&](const Frag (&fa)[MT], const Frag (&fb)[NT], int t, bool fresh) {
     const int i = t / NT, j = t % NT;
     const v16f zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-    acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(as_v8(fb[j]), as_v8(fa[i]), fresh ? zero : acc[i][j], 0, 0, 0, 0, 0, 0);
+    if (BLOCKSCALE) {
+      auto& tm = tmp[BLOCKSCALE ? i : 0][BLOCKSCALE ? j : 0];
+      tm = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(as_v8(fb[j]), as_v8(fa[i]), fresh ? zero : tm, 0, 0, 0, 0, 0, 0);
+    } else {
+      acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(as_v8(fb[j]), as_v8(fa[i]), fresh ? zero : acc[i][j], 0, 0, 0, 0, 0, 0);
+    }
   };
   // u-th of the 2*(MT+NT) LDS reads that fill fragment set (fa, fb) with K half s
   auto read_one = [&](Frag (&fa)[MT], Frag (&fb)[NT], const uint8_t* rows_a, const uint8_t* rows_b, int s, int u) {
@@ -472,11 +518,15 @@ void gemm_tiled_kernel(GemmParams p) {
 
     float sam[MT], sbv[NJP][8], bv[NJP][8];
 #pragma unroll
-    for (int i = 0; i < MT; ++i) sam[i] = p.a_scale[min(m0 + wm * WTM + i * 32 + l32, loc.m_end - 1)];
+    for (int i = 0; i < MT; ++i)
+      sam[i] = BLOCKSCALE ? 1.0f : p.a_scale[min(m0 + wm * WTM + i * 32 + l32, loc.m_end - 1)];
 #pragma unroll
     for (int jp = 0; jp < NJP; ++jp) {
       const int n = n0 + wn * WTN + jp * PASS_J * 32 + rd_col;
-      if (ALIGNED) {
+      if (BLOCKSCALE) {  // the factors were applied step by step
+#pragma unroll
+        for (int e = 0; e < 8; ++e) sbv[jp][e] = 1.0f;
+      } else if (ALIGNED) {
         const v4f s0 = *(const v4f*)(b_scale + n), s1 = *(const v4f*)(b_scale + n + 4);
 #pragma unroll
         for (int e = 0; e < 4; ++e) sbv[jp][e] = s0[e], sbv[jp][4 + e] = s1[e];
@@ -607,7 +657,8 @@ void gemm_tiled_kernel(GemmParams p) {
       ++cb.issued;
 #pragma unroll
       for (int t = 0; t < NMFMA; ++t) {
-        mfma_one(xa, xb, t, FIRST);
+        if (BLOCKSCALE) fold_block(t, FIRST);  // the previous step's block t, before it is overwritten
+        mfma_one(xa, xb, t, BLOCKSCALE || FIRST);
 #pragma unroll
         for (int l = 0; l < B_GROUPS; ++l)
           if (l * NMFMA / B_GROUPS == t) load_chunk_to_lds(chunk_src(gb, b_off[l], real), wb + NW * l * 1024);
@@ -645,6 +696,7 @@ void gemm_tiled_kernel(GemmParams p) {
       }
     }
     advance_a();
+    if (BLOCKSCALE) s_pend = step_scale(kt_c++);
   };
   auto read_first_half = [&]() {
 #pragma unroll
@@ -659,12 +711,20 @@ void gemm_tiled_kernel(GemmParams p) {
   for (int c_item = walk.slot; c_item < walk.chunk_len; c_item += walk.slots) {
     const int c_split = item_split(c_item);
     const int n_steps = split_end(c_split) - split_begin(c_split);
+    if (BLOCKSCALE) {
+      load_block_scales(locate(walk_c, c_item));
+      kt_c = split_begin(c_split);
+    }
     if (n_steps == 1) {
       step(std::true_type{}, std::false_type{});
     } else {
       step(std::true_type{}, std::true_type{});
       for (int k = 2; k < n_steps; ++k) step(std::false_type{}, std::true_type{});
       step(std::false_type{}, std::false_type{});
+    }
+    if (BLOCKSCALE) {
+#pragma unroll
+      for (int t = 0; t < NMFMA; ++t) fold_block(t, false);  // the last step's product
     }
     {
       const TileLoc loc = locate(walk_c, c_item);
@@ -1223,7 +1283,7 @@ int raise_lds_limit(const void* kernel, size_t lds_bytes, bool (&done)[kMaxDevic
   return MI355X_FP8_OK;
 }
 
-template <int BM, int BN, int WAVES_M, int WAVES_N, bool KTAIL, int EPI, bool GROUPED = false>
+template <int BM, int BN, int WAVES_M, int WAVES_N, bool KTAIL, int EPI, bool GROUPED = false, bool BLOCKSCALE = false>
 int launch_tiled(GemmParams p, hipStream_t stream) {
   constexpr int threads = WAVES_M * WAVES_N * 64;
   constexpr size_t lds_bytes = tiled_lds_bytes(BM, BN);
@@ -1232,9 +1292,9 @@ int launch_tiled(GemmParams p, hipStream_t stream) {
   p.tiles_n = (p.N + BN - 1) / BN;
   p.group_m = 4;
   const long total = (long)p.tiles_m * p.tiles_n * p.splits;
-  const long slots = (long)kNumCu * tiled_wgs_per_cu(BM, BN);
+  const long slots = (long)kNumCu * tiled_wgs_per_cu(BM, BN, BLOCKSCALE);
   long grid = total < slots ? ((total + kNumXcd - 1) / kNumXcd) * kNumXcd : slots;
-  auto kern = gemm_tiled_kernel<BM, BN, WAVES_M, WAVES_N, KTAIL, EPI, GROUPED>;
+  auto kern = gemm_tiled_kernel<BM, BN, WAVES_M, WAVES_N, KTAIL, EPI, GROUPED, BLOCKSCALE>;
   static bool attr_done[kMaxDevices] = {};
   if (const int st = raise_lds_limit((const void*)kern, lds_bytes, attr_done)) return st;
   hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(threads), lds_bytes, stream, p);
@@ -1416,6 +1476,37 @@ int mi355x_fp8_rowwise_grouped_gemm(const void* a, const void* b, const float* a
                  : launch_tiled<256, 256, 2, 2, false, kEpiPlain, true>(p, s);
   return ktail ? launch_tiled<128, 128, 2, 2, true, kEpiPlain, true>(p, s)
                : launch_tiled<128, 128, 2, 2, false, kEpiPlain, true>(p, s);
+}
+
+int mi355x_fp8_blockwise_gemm(const void* a, const void* b, const float* a_scale, const float* b_scale,
+                              void* c, int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldb,
+                              int64_t ldc, void* stream) {
+  int st = check_shape(M, N, K);
+  if (st != MI355X_FP8_OK) return st;
+  if (K > 256 * kStepK) return fail(MI355X_FP8_ENOTSUP, "block-scaled form handles K <= %d (got %lld)",
+                                    256 * kStepK, (long long)K);
+  if (!a || !b || !a_scale || !b_scale || !c) return fail(MI355X_FP8_EINVAL, "null operand pointer");
+  if (lda < K || ldb < K || ldc < N) return fail(MI355X_FP8_EINVAL, "leading dimension smaller than the row length");
+  if (lda % 16 || ldb % 16) return fail(MI355X_FP8_ENOTSUP, "lda and ldb must be multiples of 16");
+  if ((reinterpret_cast<uintptr_t>(a) & 15) || (reinterpret_cast<uintptr_t>(b) & 15))
+    return fail(MI355X_FP8_ENOTSUP, "a and b must be 16-byte aligned");
+  if ((reinterpret_cast<uintptr_t>(a_scale) & 3) || (reinterpret_cast<uintptr_t>(b_scale) & 3) ||
+      (reinterpret_cast<uintptr_t>(c) & 1))
+    return fail(MI355X_FP8_EINVAL, "misaligned scale or output pointer");
+  if (lda * 256 > (int64_t)UINT32_MAX || ldb * 256 > (int64_t)UINT32_MAX)
+    return fail(MI355X_FP8_ENOTSUP, "leading dimension too large");
+  GemmParams p;
+  p.a = (const uint8_t*)a; p.b = (const uint8_t*)b;
+  p.a_scale = a_scale; p.b_scale = b_scale;
+  p.bias = nullptr; p.c = (uint16_t*)c;
+  p.M = (int)M; p.N = (int)N; p.K = (int)K;
+  p.lda = lda; p.ldb = ldb; p.ldc = ldc;
+  p.tiles_m = p.tiles_n = 0; p.group_m = 1;
+  p.splits = 1; p.steps_per_split = k_steps_of(K); p.partial = nullptr;
+  p.m_sizes = nullptr; p.groups = 0;
+  hipStream_t s = (hipStream_t)stream;
+  return (K % kStepK) ? launch_tiled<128, 128, 2, 2, true, kEpiPlain, false, true>(p, s)
+                      : launch_tiled<128, 128, 2, 2, false, kEpiPlain, false, true>(p, s);
 }
 
 int mi355x_fp8_rowwise_quantize(const void* x, int src_type, void* xq, float* inv_scale, int64_t R,

@@ -155,6 +155,56 @@ def fp8_gemm_rowwise_grouped(
     return out
 
 
+BLOCK = 128  # rows and columns one block scale covers
+
+
+def fp8_gemm_blockwise(
+    xq: torch.Tensor,
+    wq: torch.Tensor,
+    x_scale: torch.Tensor,
+    w_scale: torch.Tensor,
+    out: Optional[torch.Tensor] = None,
+) -> torch.Tensor:
+    """Block-scaled FP8 GEMM: bf16 [M,N] = sum over 128-wide K blocks of (xq_blk @ wq_blk.T) *
+    x_scale[m // 128, kb] * w_scale[n // 128, kb].
+
+    Same operands as the callables of tritonbench/operators/fp8_gemm_blockwise/operator.py:139-145:
+    xq [M,K], wq [N,K] float8_e4m3fn; x_scale [ceil(M/128), ceil(K/128)] and w_scale
+    [ceil(N/128), ceil(K/128)] float32 as fp8_block_quantize returns them (:86-118).
+    Only enqueues work on the current stream.
+    """
+    lib = _lib.load()
+    for t, name in ((xq, "xq"), (wq, "wq"), (x_scale, "x_scale"), (w_scale, "w_scale")):
+        _require_gpu(t, name)
+    if xq.dtype != FP8_DTYPE or wq.dtype != FP8_DTYPE:
+        raise TypeError(f"xq and wq must be {FP8_DTYPE}")
+    if xq.dim() != 2 or wq.dim() != 2 or xq.shape[1] != wq.shape[1]:
+        raise ValueError("expected xq [M,K] and wq [N,K]")
+    m, k = xq.shape
+    n = wq.shape[0]
+    gm, gn, gk = -(-m // BLOCK), -(-n // BLOCK), -(-k // BLOCK)
+    if x_scale.dtype != torch.float32 or w_scale.dtype != torch.float32:
+        raise TypeError("x_scale and w_scale must be float32")
+    if tuple(x_scale.shape) != (gm, gk) or tuple(w_scale.shape) != (gn, gk):
+        raise ValueError(f"expected x_scale [{gm},{gk}] and w_scale [{gn},{gk}], got {tuple(x_scale.shape)} and {tuple(w_scale.shape)}")
+    if not x_scale.is_contiguous() or not w_scale.is_contiguous():
+        raise ValueError("scales must be contiguous")
+    if xq.stride(1) != 1 or wq.stride(1) != 1:
+        raise ValueError("xq and wq must be K-contiguous")
+    if out is None:
+        out = torch.empty((m, n), dtype=torch.bfloat16, device=xq.device)
+    else:
+        _require_gpu(out, "out")
+        if out.dtype != torch.bfloat16 or tuple(out.shape) != (m, n) or out.stride(1) != 1:
+            raise ValueError("out must be bfloat16 [M,N] with unit column stride")
+    st = lib.mi355x_fp8_blockwise_gemm(
+        xq.data_ptr(), wq.data_ptr(), x_scale.data_ptr(), w_scale.data_ptr(), out.data_ptr(),
+        m, n, k, xq.stride(0), wq.stride(0), out.stride(0), _stream_ptr(),
+    )
+    _lib.check(st, "mi355x_fp8_blockwise_gemm")
+    return out
+
+
 def fp8_row_quantize(x: torch.Tensor) -> Tuple[torch.Tensor, torch.Tensor]:
     """Row-wise e4m3fn quantisation on the GPU; returns (xq, inverse scale) like
     fp8_row_quantize in tritonbench/operators/fp8_gemm_rowwise/operator.py:136-145."""
