@@ -158,6 +158,33 @@ def time_grouped(g, m, n, k, dev, steps=40, copies=2):
                 frac=flops / ms / 1e9 / PEAK_FP8_TFLOPS)
 
 
+def time_blockwise(m, n, k, dev, steps=30):
+    """Block-scaled form (128x128 blocks of seeded N(0,1) data, quantised on the device with
+    torch ops as the reference's input generator does): flops = 2*M*N*K."""
+    from tritonbench_amd import ops
+    from tritonbench_amd.operators.fp8_gemm_blockwise.operator import fp8_block_quantize
+
+    gen = torch.Generator(device=dev)
+    gen.manual_seed(SEED + 5 * m + n + k)
+    xq, xs = fp8_block_quantize(torch.randn((m, k), generator=gen, device=dev, dtype=torch.float32))
+    wq, ws = fp8_block_quantize(torch.randn((n, k), generator=gen, device=dev, dtype=torch.float32))
+    out = torch.empty((m, n), dtype=torch.bfloat16, device=dev)
+    for _ in range(5):
+        ops.fp8_gemm_blockwise(xq, wq, xs, ws, out=out)
+    torch.cuda.synchronize()
+    stream = torch.cuda.current_stream()
+    start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    start.record(stream)
+    for _ in range(steps):
+        ops.fp8_gemm_blockwise(xq, wq, xs, ws, out=out)
+    end.record(stream)
+    torch.cuda.synchronize()
+    ms = start.elapsed_time(end) / steps
+    flops, nbytes = 2 * m * n * k, m * k + n * k + 2 * m * n
+    return dict(us=ms * 1e3, tflops=flops / ms / 1e9, gbps=nbytes / ms / 1e6, bound="mfma",
+                frac=flops / ms / 1e9 / PEAK_FP8_TFLOPS)
+
+
 def figures(m, n, k, bias, ms):
     flops = 2 * m * n * k + (2 * m * n if bias else 0)
     nbytes = m * k + n * k + 2 * m * n
@@ -289,6 +316,7 @@ def main():
         configs["c2_square_8192_graph"] = figures(m, n, k, False, time_steps_graph(sets, 20, 2))
         configs["grouped_g4_8192x4096x4096"] = time_grouped(4, 8192, 4096, 4096, dev)
         configs["grouped_g16_8192x8192x8192"] = time_grouped(16, 8192, 8192, 8192, dev, steps=20)
+        configs["blockwise_8192x8192x8192"] = time_blockwise(8192, 8192, 8192, dev)
         configs["quantise_f32_8192x8192"] = time_quantiser(8192, 8192, torch.float32, dev)
         configs["quantise_bf16_8192x8192"] = time_quantiser(8192, 8192, torch.bfloat16, dev)
         configs["quantise_bf16_57344x8192"] = time_quantiser(57344, 8192, torch.bfloat16, dev, steps=20, copies=2)

@@ -3,7 +3,7 @@
 The tritonbench checkout holds no golden vectors or known-answer tests for
 fp8_gemm_rowwise (the operator is skipped by its CI), so the vectors are produced here:
 seeded inputs, quantised by oracle.fp8_rowwise.fp8_row_quantize, outputs from
-oracle.fp8_rowwise.dequant_matmul (grouped_dequant_matmul for the grouped cases). Each .npz holds raw arrays only (uint8 e4m3fn codes,
+oracle.fp8_rowwise.dequant_matmul (grouped_dequant_matmul / blockwise_dequant_matmul for the grouped and block-scaled cases). Each .npz holds raw arrays only (uint8 e4m3fn codes,
 float32 scales, uint16 bf16 bit patterns); load with allow_pickle=False.
 
     python tests/golden/make_golden.py
@@ -35,6 +35,12 @@ GROUPED_CASES = [
     # name, g, m, n, k, sizes
     ("grouped_g3_300x72x144", 3, 300, 72, 144, [130, 0, 150]),  # an empty group; 20 rows owned by no group
     ("grouped_g2_64x33x272", 2, 64, 33, 272, None),              # equal split, N not a multiple of 4
+]
+
+
+BLOCKWISE_CASES = [
+    # name, m, n, k  (128x128 block scales)
+    ("blockwise_130x72x272", 130, 72, 272),
 ]
 
 
@@ -72,9 +78,24 @@ def main():
         np.savez_compressed(os.path.join(HERE, fname), **arrays)
         digest = hashlib.sha256(b"".join(np.ascontiguousarray(v).tobytes() for _, v in sorted(arrays.items()))).hexdigest()
         manifest["grouped_cases"].append(dict(name=name, file=fname, g=g, m=m, n=n, k=k, sha256=digest))
+    manifest["blockwise_cases"] = []
+    for name, m, n, k in BLOCKWISE_CASES:
+        xq, wq, xs, ws = orc.make_blockwise_inputs(m, n, k)
+        out = orc.blockwise_dequant_matmul(xq, wq, xs, ws)
+        arrays = dict(
+            a=xq.view(torch.uint8).numpy(),
+            b=wq.view(torch.uint8).numpy(),
+            a_scale=xs.numpy(),
+            b_scale=ws.numpy(),
+            c=out.view(torch.int16).numpy().view(np.uint16),
+        )
+        fname = name + ".npz"
+        np.savez_compressed(os.path.join(HERE, fname), **arrays)
+        digest = hashlib.sha256(b"".join(np.ascontiguousarray(v).tobytes() for _, v in sorted(arrays.items()))).hexdigest()
+        manifest["blockwise_cases"].append(dict(name=name, file=fname, m=m, n=n, k=k, sha256=digest))
     with open(os.path.join(HERE, "manifest.json"), "w") as f:
         json.dump(manifest, f, indent=1)
-    print(f"wrote {len(CASES)} + {len(GROUPED_CASES)} cases")
+    print(f"wrote {len(CASES)} + {len(GROUPED_CASES)} + {len(BLOCKWISE_CASES)} cases")
 
 
 if __name__ == "__main__":

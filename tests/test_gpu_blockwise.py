@@ -38,6 +38,24 @@ def _check_tight(out, xq, wq, xs, ws):
     assert np.all(np.abs(got - exact) <= ulp + slack), f"max excess {np.max(np.abs(got - exact) - ulp - slack)}"
 
 
+def test_blockwise_golden_fixture(gpu_device):
+    import json
+    import os
+
+    golden = os.path.join(os.path.dirname(__file__), "golden")
+    with open(os.path.join(golden, "manifest.json")) as f:
+        manifest = json.load(f)
+    for case in manifest["blockwise_cases"]:
+        z = np.load(os.path.join(golden, case["file"]), allow_pickle=False)
+        xq = torch.from_numpy(z["a"]).view(torch.float8_e4m3fn)
+        wq = torch.from_numpy(z["b"]).view(torch.float8_e4m3fn)
+        xs, ws = torch.from_numpy(z["a_scale"]), torch.from_numpy(z["b_scale"])
+        want = torch.from_numpy(z["c"].view(np.int16)).view(torch.bfloat16)
+        out = _run(gpu_device, xq, wq, xs, ws)
+        torch.testing.assert_close(out, want, rtol=RTOL, atol=ATOL)
+        _check_tight(out, xq, wq, xs, ws)
+
+
 SHAPES = [(128, 128, 128), (256, 384, 512), (1, 16, 16), (130, 260, 272), (300, 200, 2048), (127, 129, 144),
           (512, 768, 1024), (64, 4096, 2048), (1000, 520, 4112), (257, 131, 9 * 128)]
 

@@ -333,3 +333,30 @@ def test_grouped_operator_cpu_plumbing():
     assert REGISTERED_BENCHMARKS["fp8_gemm_rowwise_grouped"]["_hip_mi355x"].label == "hip_mi355x"
     with pytest.raises((RuntimeError, NotImplementedError)):
         op._hip_mi355x(group_A, group_B, m_sizes, a_scale, b_scale)()
+
+
+def test_blockwise_operator_cpu_plumbing():
+    from tritonbench_amd.harness.loader import list_operators, load_opbench_by_name
+    from tritonbench_amd.operators.fp8_gemm_blockwise import operator as bw
+
+    assert "fp8_gemm_blockwise" in list_operators()
+    Op = load_opbench_by_name("fp8_gemm_blockwise")
+    args, extra = get_parser().parse_known_args(
+        ["--op", "fp8_gemm_blockwise", "--device", "cpu", "--m", "130", "--n", "64", "--k", "272",
+         "--metrics", "latency,tflops", "--only", "_torch_dequant_cpu"])
+    op = Op(tb_args=args, extra_args=extra)
+    xq, wq, x_scale, w_scale = next(op.get_input_iter())
+    assert xq.shape == (130, 272) and x_scale.shape == (2, 3) and w_scale.shape == (1, 3)
+    # the operator's quantiser (bf16 source, any device) is the oracle's, bit for bit
+    from oracle import fp8_rowwise as orc
+    x = orc.randn_f32(130, 272, 1.0, seed=5).to(torch.bfloat16)
+    q1, s1 = bw.fp8_block_quantize(x)
+    q2, s2 = orc.fp8_block_quantize(x)
+    assert torch.equal(q1.view(torch.uint8), q2.view(torch.uint8)) and torch.equal(s1, s2)
+    want = orc.blockwise_dequant_matmul(xq, wq, x_scale, w_scale)
+    assert torch.equal(op._torch_dequant_cpu(xq, wq, x_scale, w_scale)(), want)
+    op.run(1, 2)
+    headers, table = op.output._table()
+    assert headers == ["(M, N, K)", "torch_cpu_ref-latency", "torch_cpu_ref-tflops"]
+    assert table[0][0] == (130, 64, 272)
+    assert REGISTERED_BENCHMARKS["fp8_gemm_blockwise"]["_hip_mi355x"].label == "hip_mi355x"

@@ -91,3 +91,27 @@ def test_blockwise_scales_pick_their_own_k_block():
     ws = torch.tensor([[4.0, 0.25]])
     out = orc.blockwise_dequant_matmul(xq, wq, xs, ws).float()
     assert torch.all(out == 128 * (0.5 * 4.0 + 2.0 * 0.25))
+
+
+def test_blockwise_golden_fixture_matches_oracle_and_bruteforce():
+    import json
+    import os
+
+    golden = os.path.join(os.path.dirname(__file__), "golden")
+    with open(os.path.join(golden, "manifest.json")) as f:
+        manifest = json.load(f)
+    assert manifest["blockwise_cases"]
+    for case in manifest["blockwise_cases"]:
+        z = np.load(os.path.join(golden, case["file"]), allow_pickle=False)
+        m, n, k = case["m"], case["n"], case["k"]
+        assert z["a"].shape == (m, k) and z["b"].shape == (n, k) and z["c"].shape == (m, n)
+        assert z["a_scale"].shape == (-(-m // 128), -(-k // 128)) and z["b_scale"].shape == (-(-n // 128), -(-k // 128))
+        xq = torch.from_numpy(z["a"]).view(torch.float8_e4m3fn)
+        wq = torch.from_numpy(z["b"]).view(torch.float8_e4m3fn)
+        xs, ws = torch.from_numpy(z["a_scale"]), torch.from_numpy(z["b_scale"])
+        out = orc.blockwise_dequant_matmul(xq, wq, xs, ws)
+        got_bits = out.view(torch.int16).numpy().view(np.uint16)
+        assert np.mean(got_bits == z["c"]) > 0.99, case["name"]
+        want = orc.bf16_bits_to_f32(z["c"]).astype(np.float64)
+        exact, slack = _blockwise_bruteforce(xq, wq, xs, ws)
+        assert np.all(np.abs(want - exact) <= np.abs(exact) * 2.0 ** -8 + slack), case["name"]

@@ -136,13 +136,13 @@ __device__ __forceinline__ void tile_coords(int t, int tiles_m, int tiles_n, int
 // tile's rows: 128 bytes per row = 8 chunks of 16 bytes, fetched from global memory as whole
 // 128-byte lines. Chunk c of row r sits at chunk position c ^ ((r >> 1) & 7): the MFMA
 // operand reads (consecutive lanes = consecutive rows, same logical chunk) then spread over
-// all banks. A has two stages, B three (2*32 KB + 3*32 KB = all 160 KB of a 256x256 tile's
-// LDS): the A loads of a step are the only ones that must arrive within one step, and they
-// are issued first, so at most half of every load burst is urgent.
+// all banks. With the load distance of 2 steps that every instantiation uses A has two stages,
+// B three (2*32 KB + 3*32 KB = all 160 KB of a 256x256 tile's LDS). (A distance of 4 was
+// measured on the 128x128 tile with one workgroup per CU and bought under 10 %: that tile is
+// bound by LDS bandwidth - its 64x64 wave tiles read 128 B/clk of operands - not by latency.)
 // ------------------------------------------------------------------------------------
 constexpr int kStepK = 128;
-constexpr int kStagesA = 2;
-constexpr int kStagesB = 3;
+constexpr int kDefaultDist = 2;  // steps a load runs ahead of its use; A ring = DIST stages, B ring = DIST + 1
 
 __device__ __forceinline__ int swz128(int row) { return (row >> 1) & 7; }
 
@@ -198,27 +198,32 @@ struct StepCursor {
 // SIMD (256 registers each).
 constexpr int kEpiPlain = 0, kEpiBias = 1, kEpiPartial = 2;
 
-constexpr size_t tiled_lds_bytes(int BM, int BN) { return (size_t)(kStagesA * BM + kStagesB * BN) * kStepK; }
+constexpr size_t tiled_lds_bytes(int BM, int BN, int dist = kDefaultDist) {
+  return (size_t)(dist * BM + (dist + 1) * BN) * kStepK;
+}
 // (the block-scaled form keeps a second accumulator set and needs the whole register file)
-constexpr int tiled_wgs_per_cu(int BM, int BN, bool blockscale = false) {
-  return !blockscale && tiled_lds_bytes(BM, BN) <= 80 * 1024 ? 2 : 1;
+constexpr int tiled_wgs_per_cu(int BM, int BN, bool blockscale = false, int dist = kDefaultDist) {
+  return !blockscale && tiled_lds_bytes(BM, BN, dist) <= 80 * 1024 ? 2 : 1;
 }
 
 //
 // BLOCKSCALE turns the kernel into the 128x128x128 block-scaled GEMM: a_scale is then
 // [ceil(M/128)][ceil(K/128)], b_scale [ceil(N/128)][ceil(K/128)], and every K step's product
-// is multiplied by a_scale[mb][kb] * b_scale[nb][kb] before it is added up. With 128x128 tiles
-// and 128-byte steps that factor is one number per workgroup and step: the MFMAs of a step
+// is multiplied by a_scale[mb][kb] * b_scale[nb][kb] before it is added up. With wave tiles
+// inside one scale block and 128-byte steps that factor is one number per wave and step: the MFMAs of a step
 // go to a second accumulator set, which is folded into the first (acc += s * tmp) behind
 // the next step's MFMAs.
-template <int BM, int BN, int WAVES_M, int WAVES_N, bool KTAIL, int EPI, bool GROUPED = false, bool BLOCKSCALE = false>
+template <int BM, int BN, int WAVES_M, int WAVES_N, bool KTAIL, int EPI, bool GROUPED = false, bool BLOCKSCALE = false,
+          int DIST = kDefaultDist>
 __global__ __launch_bounds__(WAVES_M* WAVES_N * 64)
-__attribute__((amdgpu_waves_per_eu(tiled_wgs_per_cu(BM, BN, BLOCKSCALE) * WAVES_M * WAVES_N / 4,
-                                   tiled_wgs_per_cu(BM, BN, BLOCKSCALE) * WAVES_M * WAVES_N / 4)))
+__attribute__((amdgpu_waves_per_eu(tiled_wgs_per_cu(BM, BN, BLOCKSCALE, DIST) * WAVES_M * WAVES_N / 4,
+                                   tiled_wgs_per_cu(BM, BN, BLOCKSCALE, DIST) * WAVES_M * WAVES_N / 4)))
 void gemm_tiled_kernel(GemmParams p) {
+  constexpr int kStagesA = DIST, kStagesB = DIST + 1;
+  static_assert(DIST >= 2 && tiled_lds_bytes(BM, BN, DIST) <= 160 * 1024, "the stage rings must fit the LDS");
   static_assert(!GROUPED || EPI == kEpiPlain, "the grouped form has neither bias nor split-K");
-  static_assert(!BLOCKSCALE || (BM == 128 && BN == 128 && EPI == kEpiPlain && !GROUPED),
-                "block scales are per 128x128 tile: one tile, one scale per step");
+  static_assert(!BLOCKSCALE || (128 % (BM / WAVES_M) == 0 && 128 % (BN / WAVES_N) == 0 && EPI == kEpiPlain && !GROUPED),
+                "a wave's tile must lie inside one 128x128 scale block: one factor per wave and step");
   constexpr bool HAS_BIAS = EPI == kEpiBias;
   constexpr int NW = WAVES_M * WAVES_N;
   constexpr int WTM = BM / WAVES_M;    // wave tile rows (m)
@@ -230,7 +235,7 @@ void gemm_tiled_kernel(GemmParams p) {
   constexpr int B_GROUPS = BN / 8 / NW;
   static_assert(BM % (8 * NW) == 0 && BN % (8 * NW) == 0, "tile rows must split over waves");
   static_assert(WTM % 32 == 0 && WTN % 32 == 0, "wave tile must be a multiple of 32x32");
-  static_assert(A_GROUPS + 2 * B_GROUPS < 64, "outstanding-load count must fit the vmcnt field");
+  static_assert(DIST * (A_GROUPS + B_GROUPS) < 64, "outstanding-load count must fit the vmcnt field");
 
   extern __shared__ __attribute__((aligned(1024))) uint8_t lds[];
 
@@ -413,8 +418,10 @@ void gemm_tiled_kernel(GemmParams p) {
   constexpr int SC_REGS = 4;  // 256 steps = K up to 32768
   float sc[SC_REGS] = {0.f, 0.f, 0.f, 0.f};
   auto load_block_scales = [&](const TileLoc& loc) {
-    const float* sa = p.a_scale + (size_t)(loc.m0 / 128) * k_steps;
-    const float* sb = p.b_scale + (size_t)(loc.n0 / 128) * k_steps;
+    // the scale block of this wave's tile (clamped for waves that lie past the matrix edge)
+    const int mb = min(loc.m0 + wm * WTM, p.M - 1) / 128, nb = min(loc.n0 + wn * WTN, p.N - 1) / 128;
+    const float* sa = p.a_scale + (size_t)mb * k_steps;
+    const float* sb = p.b_scale + (size_t)nb * k_steps;
 #pragma unroll
     for (int r = 0; r < SC_REGS; ++r) {
       const int kb = min(r * 64 + lane, k_steps - 1);
@@ -466,14 +473,15 @@ void gemm_tiled_kernel(GemmParams p) {
   constexpr int RPS = (NREAD + NMFMA / 2 - 1) / (NMFMA / 2);
   static_assert(A_GROUPS <= NMFMA && B_GROUPS <= NMFMA, "at most one load slot per MFMA");
 
-  // ---- prologue: A(0) B(0) A(1) B(1) in flight, first fragments in registers
+  // ---- prologue: A(0) B(0) .. A(DIST-1) B(DIST-1) in flight, first fragments in registers
   setup_a(ca.item);
   setup_b(cb.item);
-  issue_a(); advance_a();
-  issue_b(); advance_b();
-  issue_a(); advance_a();
-  issue_b(); advance_b();
-  wait_loads_and_barrier<A_GROUPS + B_GROUPS>();
+#pragma unroll
+  for (int d = 0; d < DIST; ++d) {
+    issue_a(); advance_a();
+    issue_b(); advance_b();
+  }
+  wait_loads_and_barrier<(DIST - 1) * (A_GROUPS + B_GROUPS)>();
 #pragma unroll
   for (int u = 0; u < NREAD; ++u) read_one(xa, xb, lds + a_rd_base, lds + b_rd_base, 0, u);
 
@@ -646,7 +654,7 @@ void gemm_tiled_kernel(GemmParams p) {
 
     // [A] MFMAs on x* (first K half of this step). Behind them, one per MFMA: the LDS reads
     //     of the second half (-> y*), and behind every other one a global->LDS load of
-    //     B(g+2) into the B stage released at the previous barrier. The fences pin this
+    //     B(g+DIST) into the B stage released at the previous barrier. The fences pin this
     //     interleaving: every wave-level memory instruction hides behind an MFMA, and the
     //     load queue never holds more than the matrix pipe can cover.
     __builtin_amdgcn_sched_barrier(0);
@@ -670,11 +678,12 @@ void gemm_tiled_kernel(GemmParams p) {
     }
     advance_b();
 
-    // own loads of A(g+1) and B(g+1) have landed (B(g+2) may still be in flight); past the
-    // barrier everyone's have, and every wave is done reading this step's stages
-    wait_loads_and_barrier<B_GROUPS>();
+    // own loads of A(g+1) and B(g+1) have landed (the younger B(g+2) .. B(g+DIST) and
+    // A(g+2) .. A(g+DIST-1) may still be in flight); past the barrier everyone's have, and
+    // every wave is done reading this step's stages
+    wait_loads_and_barrier<(DIST - 1) * B_GROUPS + (DIST - 2) * A_GROUPS>();
 
-    // [B] MFMAs on y* (second K half); behind them the loads of A(g+2) into the A stage just
+    // [B] MFMAs on y* (second K half); behind them the loads of A(g+DIST) into the A stage just
     //     released and the LDS reads of step g+1's first half (-> x*; at the end of a tile
     //     these already belong to the next tile)
     __builtin_amdgcn_sched_barrier(0);
@@ -1283,18 +1292,19 @@ int raise_lds_limit(const void* kernel, size_t lds_bytes, bool (&done)[kMaxDevic
   return MI355X_FP8_OK;
 }
 
-template <int BM, int BN, int WAVES_M, int WAVES_N, bool KTAIL, int EPI, bool GROUPED = false, bool BLOCKSCALE = false>
+template <int BM, int BN, int WAVES_M, int WAVES_N, bool KTAIL, int EPI, bool GROUPED = false, bool BLOCKSCALE = false,
+          int DIST = kDefaultDist>
 int launch_tiled(GemmParams p, hipStream_t stream) {
   constexpr int threads = WAVES_M * WAVES_N * 64;
-  constexpr size_t lds_bytes = tiled_lds_bytes(BM, BN);
+  constexpr size_t lds_bytes = tiled_lds_bytes(BM, BN, DIST);
   // grouped: the group sizes live on the device; every group adds at most one partial tile row
   p.tiles_m = GROUPED ? p.M / BM + p.groups : (p.M + BM - 1) / BM;
   p.tiles_n = (p.N + BN - 1) / BN;
   p.group_m = 4;
   const long total = (long)p.tiles_m * p.tiles_n * p.splits;
-  const long slots = (long)kNumCu * tiled_wgs_per_cu(BM, BN, BLOCKSCALE);
+  const long slots = (long)kNumCu * tiled_wgs_per_cu(BM, BN, BLOCKSCALE, DIST);
   long grid = total < slots ? ((total + kNumXcd - 1) / kNumXcd) * kNumXcd : slots;
-  auto kern = gemm_tiled_kernel<BM, BN, WAVES_M, WAVES_N, KTAIL, EPI, GROUPED, BLOCKSCALE>;
+  auto kern = gemm_tiled_kernel<BM, BN, WAVES_M, WAVES_N, KTAIL, EPI, GROUPED, BLOCKSCALE, DIST>;
   static bool attr_done[kMaxDevices] = {};
   if (const int st = raise_lds_limit((const void*)kern, lds_bytes, attr_done)) return st;
   hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(threads), lds_bytes, stream, p);
@@ -1309,17 +1319,17 @@ int launch_tiled(GemmParams p, hipStream_t stream) {
   return MI355X_FP8_OK;
 }
 
-template <int BM, int BN, int WAVES_M, int WAVES_N>
+template <int BM, int BN, int WAVES_M, int WAVES_N, int DIST = kDefaultDist>
 int launch_tiled_config(const GemmParams& p, hipStream_t s) {
   const bool ktail = p.K % kStepK;
   if (p.splits > 1)
-    return ktail ? launch_tiled<BM, BN, WAVES_M, WAVES_N, true, kEpiPartial>(p, s)
-                 : launch_tiled<BM, BN, WAVES_M, WAVES_N, false, kEpiPartial>(p, s);
+    return ktail ? launch_tiled<BM, BN, WAVES_M, WAVES_N, true, kEpiPartial, false, false, DIST>(p, s)
+                 : launch_tiled<BM, BN, WAVES_M, WAVES_N, false, kEpiPartial, false, false, DIST>(p, s);
   if (p.bias)
-    return ktail ? launch_tiled<BM, BN, WAVES_M, WAVES_N, true, kEpiBias>(p, s)
-                 : launch_tiled<BM, BN, WAVES_M, WAVES_N, false, kEpiBias>(p, s);
-  return ktail ? launch_tiled<BM, BN, WAVES_M, WAVES_N, true, kEpiPlain>(p, s)
-               : launch_tiled<BM, BN, WAVES_M, WAVES_N, false, kEpiPlain>(p, s);
+    return ktail ? launch_tiled<BM, BN, WAVES_M, WAVES_N, true, kEpiBias, false, false, DIST>(p, s)
+                 : launch_tiled<BM, BN, WAVES_M, WAVES_N, false, kEpiBias, false, false, DIST>(p, s);
+  return ktail ? launch_tiled<BM, BN, WAVES_M, WAVES_N, true, kEpiPlain, false, false, DIST>(p, s)
+               : launch_tiled<BM, BN, WAVES_M, WAVES_N, false, kEpiPlain, false, false, DIST>(p, s);
 }
 
 template <int MT, int NTW, int DEPTH, int KW>
@@ -1505,6 +1515,8 @@ int mi355x_fp8_blockwise_gemm(const void* a, const void* b, const float* a_scale
   p.splits = 1; p.steps_per_split = k_steps_of(K); p.partial = nullptr;
   p.m_sizes = nullptr; p.groups = 0;
   hipStream_t s = (hipStream_t)stream;
+  // 128x128 tiles: with 256x128 tiles (64 more accumulators and 64 more partial products per
+  // lane) the fold no longer fits the 256 registers VALU instructions can address
   return (K % kStepK) ? launch_tiled<128, 128, 2, 2, true, kEpiPlain, false, true>(p, s)
                       : launch_tiled<128, 128, 2, 2, false, kEpiPlain, false, true>(p, s);
 }
