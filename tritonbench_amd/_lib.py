@@ -22,7 +22,7 @@ VARIANT_AUTO = 0
 VARIANT_TILED = 1
 VARIANT_SKINNY = 2
 
-NUM_TILE_CONFIGS = 2
+NUM_TILE_CONFIGS = 3
 
 
 def tiled_variant(config=None, splits=0) -> int:

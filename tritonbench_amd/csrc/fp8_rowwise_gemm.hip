@@ -1207,11 +1207,12 @@ struct TileConfig {
   float us_per_item;        // pipeline refill + epilogue of one work item
   float stream_bytes_per_us;  // operand bytes per microsecond the configuration can stream from HBM
 };
-constexpr int kNumTileConfigs = 2;
+constexpr int kNumTileConfigs = 3;
 // Measured on MI355X with normally distributed operands (clock under sustained MFMA load).
 constexpr TileConfig kTileConfigs[kNumTileConfigs] = {
     {256, 256, tiled_wgs_per_cu(256, 256), 1.30f, 1.30f, 6.0f, 3.6e6f},
     {128, 128, tiled_wgs_per_cu(128, 128), 1.00f, 0.62f, 5.0f, 4.4e6f},
+    {256, 128, tiled_wgs_per_cu(256, 128), 0.87f, 0.87f, 5.0f, 4.0e6f},
 };
 constexpr int kMaxSplits = 16;
 
@@ -1428,6 +1429,7 @@ int mi355x_fp8_rowwise_gemm(const void* a, const void* b, const float* a_scale, 
         switch (plan.config) {
           case 0: return launch_tiled_config<256, 256, 2, 2>(p, s);
           case 1: return launch_tiled_config<128, 128, 2, 2>(p, s);
+          case 2: return launch_tiled_config<256, 128, 2, 2>(p, s);
           default: return fail(MI355X_FP8_EINVAL, "unknown tile configuration %d", plan.config);
         }
       }
@@ -1484,6 +1486,9 @@ int mi355x_fp8_rowwise_grouped_gemm(const void* a, const void* b, const float* a
   if (tile_config == 0)
     return ktail ? launch_tiled<256, 256, 2, 2, true, kEpiPlain, true>(p, s)
                  : launch_tiled<256, 256, 2, 2, false, kEpiPlain, true>(p, s);
+  if (tile_config == 2)
+    return ktail ? launch_tiled<256, 128, 2, 2, true, kEpiPlain, true>(p, s)
+                 : launch_tiled<256, 128, 2, 2, false, kEpiPlain, true>(p, s);
   return ktail ? launch_tiled<128, 128, 2, 2, true, kEpiPlain, true>(p, s)
                : launch_tiled<128, 128, 2, 2, false, kEpiPlain, true>(p, s);
 }
