@@ -157,11 +157,6 @@ __device__ __forceinline__ void load_chunk_to_lds(const uint8_t* gsrc, uint8_t* 
 // read as zeros (whatever follows a row in memory could decode to NaN).
 __device__ const v4i kZeroChunk = {0, 0, 0, 0};
 
-// Scheduling hints for the machine scheduler: MFMA / LDS read / global load slots.
-#define SCHED_MFMA(n) __builtin_amdgcn_sched_group_barrier(0x008, n, 0)
-#define SCHED_DSREAD(n) __builtin_amdgcn_sched_group_barrier(0x100, n, 0)
-#define SCHED_VMEM(n) __builtin_amdgcn_sched_group_barrier(0x020, n, 0)
-
 // Waits until at most VM of this wave's global loads and none of its LDS operations are
 // outstanding, then joins the workgroup barrier. Written with the s_waitcnt builtin (not
 // inline asm) so the compiler's own wait-count bookkeeping knows the LDS queue is empty
@@ -181,13 +176,14 @@ struct StepCursor {
 };
 
 // The kernel is one software pipeline over "steps" (a 128-byte K slab of one tile) that runs
-// through all tiles a workgroup owns without draining at tile boundaries. For step g:
+// through all tiles a workgroup owns without draining at tile boundaries. For step g, with
+// loads running DIST (= 2) steps ahead:
 //
 //   [A] MFMAs of (g, first K half), interleaved with the LDS reads of (g, second half) and
-//       the loads of B(g+2) (its stage was released at the previous barrier)
+//       the loads of B(g+DIST) (its stage was released at the previous barrier)
 //       wait for own loads of A(g+1) and B(g+1); workgroup barrier
 //   [B] MFMAs of (g, second half), interleaved with the LDS reads of (g+1, first half) and
-//       the loads of A(g+2) into the A stage step g just released
+//       the loads of A(g+DIST) into the A stage step g just released
 //   after a tile's last step: epilogue (loads of the next tile are already in flight)
 //
 // Two register sets of operand fragments alternate between the halves; one barrier per step.
@@ -207,12 +203,14 @@ constexpr int tiled_wgs_per_cu(int BM, int BN, bool blockscale = false, int dist
 }
 
 //
+// GROUPED walks the tiles of a stack of row blocks whose sizes are read from device memory.
+//
 // BLOCKSCALE turns the kernel into the 128x128x128 block-scaled GEMM: a_scale is then
 // [ceil(M/128)][ceil(K/128)], b_scale [ceil(N/128)][ceil(K/128)], and every K step's product
 // is multiplied by a_scale[mb][kb] * b_scale[nb][kb] before it is added up. With wave tiles
-// inside one scale block and 128-byte steps that factor is one number per wave and step: the MFMAs of a step
-// go to a second accumulator set, which is folded into the first (acc += s * tmp) behind
-// the next step's MFMAs.
+// inside one scale block and 128-byte steps that factor is one number per wave and step:
+// the MFMAs of a step go to a second accumulator set, which is folded into the first
+// (acc += s * tmp) behind the next step's MFMAs.
 template <int BM, int BN, int WAVES_M, int WAVES_N, bool KTAIL, int EPI, bool GROUPED = false, bool BLOCKSCALE = false,
           int DIST = kDefaultDist>
 __global__ __launch_bounds__(WAVES_M* WAVES_N * 64)
