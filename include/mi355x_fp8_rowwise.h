@@ -49,14 +49,15 @@ extern "C" {
 /* Kernel families. AUTO lets the library pick from (M, N, K). */
 #define MI355X_FP8_VARIANT_AUTO    0
 #define MI355X_FP8_VARIANT_TILED   1  /* LDS-tiled persistent MFMA kernel (compute-bound shapes) */
-#define MI355X_FP8_VARIANT_SKINNY  2  /* in-workgroup split-K streaming kernel (M <= 64, HBM-bound) */
+#define MI355X_FP8_VARIANT_SKINNY  2  /* in-workgroup split-K streaming kernel (M <= 64 only, HBM-bound) */
 
 /*
  * The `variant` argument is a word: bits 0..7 hold the family above; for the tiled family
  * bits 8..15 may pin the tile configuration and bits 16..23 the split-K factor (0 in a
  * field = chosen by the library from the shape). Tile configurations: 0 = 256x256 tiles,
  * one workgroup per CU; 1 = 128x128 tiles, two workgroups per CU; 2 = 256x128 tiles
- * (256 rows of A, 128 rows of B), one workgroup per CU. With a split-K factor
+ * (256 rows of A, 128 rows of B), one workgroup per CU; 3 = 64x256 tiles, one workgroup
+ * per CU (not available in the grouped form). With a split-K factor
  * S > 1 every tile's K range is cut into S parts that run as separate work items; they
  * leave fp32 partial sums in the workspace (S*M*N*4 bytes) and a second kernel adds them
  * in a fixed order, so results do not depend on scheduling. A split factor larger than the
@@ -64,7 +65,8 @@ extern "C" {
  */
 #define MI355X_FP8_TILED_CONFIG(cfg)    ((((cfg) + 1) & 0xff) << 8)
 #define MI355X_FP8_TILED_SPLITS(s)      (((s) & 0xff) << 16)
-#define MI355X_FP8_NUM_TILE_CONFIGS     3
+#define MI355X_FP8_NUM_TILE_CONFIGS     4
+#define MI355X_FP8_NUM_GROUPED_TILE_CONFIGS 3
 
 /* Source element types accepted by the quantiser. */
 #define MI355X_FP8_SRC_F32   0

@@ -42,6 +42,8 @@ def test_host_side_argument_checks_need_no_gpu():
     # shape checks happen before anything touches a device
     assert lib.mi355x_fp8_rowwise_select_variant(16, 8192, 8192) == _lib.VARIANT_SKINNY
     assert lib.mi355x_fp8_rowwise_select_variant(8192, 8192, 8192) == _lib.VARIANT_TILED
+    assert lib.mi355x_fp8_rowwise_select_variant(64, 8192, 8192) == _lib.VARIANT_SKINNY
+    assert lib.mi355x_fp8_rowwise_select_variant(64, 57344, 8192) == _lib.VARIANT_TILED
     assert lib.mi355x_fp8_rowwise_select_variant(0, 8, 16) == _lib.EINVAL
     assert lib.mi355x_fp8_rowwise_select_variant(8, 8, 24) == _lib.ENOTSUP
     assert "multiple of 16" in _lib.last_error()
@@ -67,6 +69,7 @@ def test_workspace_size_follows_the_plan_without_a_gpu():
     ws = lib.mi355x_fp8_rowwise_workspace_bytes
     text = open(HEADER).read()
     assert int(re.search(r"#define\s+MI355X_FP8_NUM_TILE_CONFIGS\s+(\d+)", text).group(1)) == _lib.NUM_TILE_CONFIGS
+    assert int(re.search(r"#define\s+MI355X_FP8_NUM_GROUPED_TILE_CONFIGS\s+(\d+)", text).group(1)) == _lib.NUM_GROUPED_TILE_CONFIGS
     # enough tiles to fill the chip, or the on-chip reduction of the skinny kernel: no workspace
     assert ws(8192, 8192, 8192, _lib.VARIANT_AUTO) == 0
     assert ws(16, 8192, 8192, _lib.VARIANT_AUTO) == 0

@@ -61,7 +61,7 @@ def test_grouped_golden_fixtures(gpu_device):
         wq = torch.from_numpy(z["b"]).view(torch.float8_e4m3fn)
         ms, xs, ws = torch.from_numpy(z["m_sizes"]), torch.from_numpy(z["a_scale"]), torch.from_numpy(z["b_scale"])
         want = torch.from_numpy(z["c"].view(np.int16)).view(torch.bfloat16)
-        for cfg in [-1] + list(range(_lib.NUM_TILE_CONFIGS)):
+        for cfg in [-1] + list(range(_lib.NUM_GROUPED_TILE_CONFIGS)):
             print(f"golden {case['name']} tile_config {cfg}", flush=True)
             out = _run(gpu_device, xq, wq, ms, xs, ws, cfg)  # allocated by the call: unowned rows are zero
             _check(out, want, (xq, wq, ms, xs, ws))
@@ -81,7 +81,7 @@ CASES = [
 
 
 @pytest.mark.parametrize("g,m,n,k,sizes", CASES)
-@pytest.mark.parametrize("tile_config", [-1] + list(range(_lib.NUM_TILE_CONFIGS)))
+@pytest.mark.parametrize("tile_config", [-1] + list(range(_lib.NUM_GROUPED_TILE_CONFIGS)))
 def test_grouped_against_oracle(gpu_device, g, m, n, k, sizes, tile_config):
     print(f"case g={g} m={m} n={n} k={k} sizes={sizes} tile_config={tile_config}", flush=True)
     xq, wq, ms, xs, ws = orc.make_grouped_inputs(g, m, n, k, sizes=sizes)
@@ -93,7 +93,7 @@ def test_grouped_against_oracle(gpu_device, g, m, n, k, sizes, tile_config):
     assert torch.all(out[covered:] == -77.0)  # rows no group owns are not written
 
 
-@pytest.mark.parametrize("tile_config", range(_lib.NUM_TILE_CONFIGS))
+@pytest.mark.parametrize("tile_config", range(_lib.NUM_GROUPED_TILE_CONFIGS))
 def test_grouped_sizes_that_lie_are_cut_off_inside_the_matrices(gpu_device, tile_config):
     # the kernel reads the sizes, the host never does: negative entries count as empty and the
     # running sum stops at M, so nothing outside A and C is touched whatever the entries say
@@ -109,7 +109,7 @@ def test_grouped_sizes_that_lie_are_cut_off_inside_the_matrices(gpu_device, tile
     assert torch.all(buf[m:] == -77.0)
 
 
-@pytest.mark.parametrize("tile_config", range(_lib.NUM_TILE_CONFIGS))
+@pytest.mark.parametrize("tile_config", range(_lib.NUM_GROUPED_TILE_CONFIGS))
 def test_grouped_exact_integer_case_is_bit_exact(gpu_device, tile_config):
     rng = np.random.default_rng(21)
     ints = np.array([0, 1, 2, 3, 4, -1, -2, -3, -4, 0.5, -0.5], dtype=np.float32)
@@ -131,7 +131,7 @@ def test_grouped_exact_integer_case_is_bit_exact(gpu_device, tile_config):
 def test_grouped_with_one_group_equals_the_plain_kernel_bit_for_bit(gpu_device):
     m, n, k = 600, 520, 768
     xq, wq, ms, xs, ws = orc.make_grouped_inputs(1, m, n, k)
-    for cfg in range(_lib.NUM_TILE_CONFIGS):
+    for cfg in range(_lib.NUM_GROUPED_TILE_CONFIGS):
         grouped = _run(gpu_device, xq, wq, ms, xs, ws, cfg)
         plain = ops.fp8_gemm_rowwise(xq.to(gpu_device), wq.to(gpu_device), xs.to(gpu_device), ws.to(gpu_device),
                                      variant=_lib.tiled_variant(cfg, 1)).cpu()
@@ -180,6 +180,6 @@ def test_grouped_invalid_arguments_raise(gpu_device):
     with pytest.raises(RuntimeError, match="no CPU fallback"):
         ops.fp8_gemm_rowwise_grouped(xq, wq, ms.cpu(), xs, ws)
     with pytest.raises(ValueError, match="tile configuration"):
-        ops.fp8_gemm_rowwise_grouped(xq, wq, ms, xs, ws, tile_config=_lib.NUM_TILE_CONFIGS)
+        ops.fp8_gemm_rowwise_grouped(xq, wq, ms, xs, ws, tile_config=_lib.NUM_GROUPED_TILE_CONFIGS)
     with pytest.raises(NotImplementedError, match="multiple of 16"):
         ops.fp8_gemm_rowwise_grouped(xq[:, :24], wq[:, :24], ms, xs, ws)

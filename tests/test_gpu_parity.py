@@ -311,6 +311,9 @@ def test_dispatch_is_pinned(gpu_device):
     assert ops.select_variant(16, 8192, 8192) == _lib.VARIANT_SKINNY
     assert ops.select_variant(64, 8192, 8192) == _lib.VARIANT_SKINNY
     assert ops.select_variant(8192, 8192, 8192) == _lib.VARIANT_TILED
+    # M <= 64 with a long weight panel and four 16-row blocks of A: 64-row tiles win
+    assert ops.select_variant(64, 57344, 8192) == _lib.VARIANT_TILED
+    assert ops.select_variant(16, 57344, 8192) == _lib.VARIANT_SKINNY
 
 
 def test_graph_capture_replays_match_eager(gpu_device):

@@ -22,7 +22,8 @@ VARIANT_AUTO = 0
 VARIANT_TILED = 1
 VARIANT_SKINNY = 2
 
-NUM_TILE_CONFIGS = 3
+NUM_TILE_CONFIGS = 4
+NUM_GROUPED_TILE_CONFIGS = 3
 
 
 def tiled_variant(config=None, splits=0) -> int:

@@ -469,7 +469,6 @@ void gemm_tiled_kernel(GemmParams p) {
   // the fragments of the next half) costs the matrix pipe nothing.
   constexpr int NMFMA = MT * NT, NREAD = 2 * (MT + NT);
   constexpr int RPS = (NREAD + NMFMA / 2 - 1) / (NMFMA / 2);
-  static_assert(A_GROUPS <= NMFMA && B_GROUPS <= NMFMA, "at most one load slot per MFMA");
 
   // ---- prologue: A(0) B(0) .. A(DIST-1) B(DIST-1) in flight, first fragments in registers
   setup_a(ca.item);
@@ -1205,17 +1204,29 @@ struct TileConfig {
   float us_per_item;        // pipeline refill + epilogue of one work item
   float stream_bytes_per_us;  // operand bytes per microsecond the configuration can stream from HBM
 };
-constexpr int kNumTileConfigs = 3;
+constexpr int kNumTileConfigs = 4;
+constexpr int kNumGroupedTileConfigs = 3;  // the grouped form uses the first three
 // Measured on MI355X with normally distributed operands (clock under sustained MFMA load).
 constexpr TileConfig kTileConfigs[kNumTileConfigs] = {
     {256, 256, tiled_wgs_per_cu(256, 256), 1.30f, 1.30f, 6.0f, 3.6e6f},
     {128, 128, tiled_wgs_per_cu(128, 128), 1.00f, 0.62f, 5.0f, 4.4e6f},
     {256, 128, tiled_wgs_per_cu(256, 128), 0.87f, 0.87f, 5.0f, 4.0e6f},
+    {64, 256, tiled_wgs_per_cu(64, 256), 0.75f, 0.75f, 7.0f, 4.8e6f},
 };
+
+// The skinny kernel's run time for comparison with the tiled plans at M <= 64: a fixed part
+// plus B streamed at a rate that falls with the number of 16-row blocks of A every workgroup
+// has to pull through L1 beside its rows of B (measured, MB per microsecond).
+inline float skinny_cost_us(int64_t M, int64_t N, int64_t K) {
+  static const float rate[4] = {7.0e6f, 5.4e6f, 4.5e6f, 4.0e6f};
+  const int blocks = (int)((M + 15) / 16);
+  return 6.0f + (float)N * (float)K / rate[blocks < 1 ? 0 : blocks > 4 ? 3 : blocks - 1];
+}
 constexpr int kMaxSplits = 16;
 
 struct TiledPlan {
   int config, splits, steps_per_split;
+  float cost_us;
 };
 
 inline int k_steps_of(int64_t K) { return (int)((K + kStepK - 1) / kStepK); }
@@ -1250,7 +1261,7 @@ inline float plan_cost_us(int64_t M, int64_t N, int64_t K, int config, int split
 inline TiledPlan plan_tiled(int64_t M, int64_t N, int64_t K, int force_config, int force_splits,
                             int max_splits) {
   const int k_steps = k_steps_of(K);
-  TiledPlan best = {0, 1, k_steps};
+  TiledPlan best = {0, 1, k_steps, 0.0f};
   float best_cost = -1.0f;
   for (int c = 0; c < kNumTileConfigs; ++c) {
     if (force_config >= 0 && c != force_config) continue;
@@ -1262,7 +1273,7 @@ inline TiledPlan plan_tiled(int64_t M, int64_t N, int64_t K, int force_config, i
       const float cost = plan_cost_us(M, N, K, c, splits, sps);
       if (best_cost < 0.0f || cost < best_cost) {
         best_cost = cost;
-        best = {c, splits, sps};
+        best = {c, splits, sps, cost};
       }
     }
   }
@@ -1356,7 +1367,11 @@ const char* mi355x_fp8_rowwise_last_error(void) { return g_err; }
 int mi355x_fp8_rowwise_select_variant(int64_t M, int64_t N, int64_t K) {
   const int st = check_shape(M, N, K);
   if (st != MI355X_FP8_OK) return st;
-  return M <= kSkinnyMaxM ? MI355X_FP8_VARIANT_SKINNY : MI355X_FP8_VARIANT_TILED;
+  // M <= 64: the streaming kernel, unless a tiled plan (64-row tiles, split K) is expected to
+  // beat it: long weight panels with three or four 16-row blocks of A
+  if (M > kSkinnyMaxM) return MI355X_FP8_VARIANT_TILED;
+  return plan_tiled(M, N, K, -1, 0, kMaxSplits).cost_us < skinny_cost_us(M, N, K) ? MI355X_FP8_VARIANT_TILED
+                                                                                 : MI355X_FP8_VARIANT_SKINNY;
 }
 
 size_t mi355x_fp8_rowwise_workspace_bytes(int64_t M, int64_t N, int64_t K, int variant) {
@@ -1388,7 +1403,17 @@ int mi355x_fp8_rowwise_gemm(const void* a, const void* b, const float* a_scale, 
     return fail(MI355X_FP8_EINVAL, "unknown variant 0x%x", variant);
   const int plan_bits = variant & ~0xff;
   variant &= 0xff;
-  if (variant == MI355X_FP8_VARIANT_AUTO) variant = mi355x_fp8_rowwise_select_variant(M, N, K);
+  if (variant == MI355X_FP8_VARIANT_AUTO) {
+    variant = mi355x_fp8_rowwise_select_variant(M, N, K);
+    if (variant == MI355X_FP8_VARIANT_TILED && M <= kSkinnyMaxM) {
+      // the choice assumed the plan's workspace; without it the plan changes and may lose
+      const TiledPlan plan = plan_from_variant(M, N, K, plan_bits, kMaxSplits);
+      const size_t need = plan.splits > 1 ? (size_t)plan.splits * M * N * sizeof(float) : 0;
+      if (need && (!workspace || workspace_bytes < need) &&
+          plan_from_variant(M, N, K, plan_bits, 1).cost_us >= skinny_cost_us(M, N, K))
+        variant = MI355X_FP8_VARIANT_SKINNY;
+    }
+  }
   if (variant == MI355X_FP8_VARIANT_SKINNY && M > kSkinnyMaxM)
     return fail(MI355X_FP8_ENOTSUP, "skinny variant handles M <= %d (got %lld)", kSkinnyMaxM, (long long)M);
 
@@ -1428,6 +1453,7 @@ int mi355x_fp8_rowwise_gemm(const void* a, const void* b, const float* a_scale, 
           case 0: return launch_tiled_config<256, 256, 2, 2>(p, s);
           case 1: return launch_tiled_config<128, 128, 2, 2>(p, s);
           case 2: return launch_tiled_config<256, 128, 2, 2>(p, s);
+          case 3: return launch_tiled_config<64, 256, 1, 4>(p, s);
           default: return fail(MI355X_FP8_EINVAL, "unknown tile configuration %d", plan.config);
         }
       }
@@ -1463,7 +1489,7 @@ int mi355x_fp8_rowwise_grouped_gemm(const void* a, const void* b, const float* a
     return fail(MI355X_FP8_EINVAL, "misaligned scale, size or output pointer (b_scale needs 16 bytes)");
   if (lda * 256 > (int64_t)UINT32_MAX || ldb * 256 > (int64_t)UINT32_MAX)
     return fail(MI355X_FP8_ENOTSUP, "leading dimension too large");
-  if (tile_config < -1 || tile_config >= kNumTileConfigs)
+  if (tile_config < -1 || tile_config >= kNumGroupedTileConfigs)
     return fail(MI355X_FP8_EINVAL, "unknown tile configuration %d", tile_config);
 
   GemmParams p;
