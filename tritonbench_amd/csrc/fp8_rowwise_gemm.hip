@@ -1218,7 +1218,7 @@ constexpr TileConfig kTileConfigs[kNumTileConfigs] = {
 // plus B streamed at a rate that falls with the number of 16-row blocks of A every workgroup
 // has to pull through L1 beside its rows of B (measured, MB per microsecond).
 inline float skinny_cost_us(int64_t M, int64_t N, int64_t K) {
-  static const float rate[4] = {7.0e6f, 5.4e6f, 4.5e6f, 4.0e6f};
+  static const float rate[4] = {7.0e6f, 4.5e6f, 4.2e6f, 3.9e6f};
   const int blocks = (int)((M + 15) / 16);
   return 6.0f + (float)N * (float)K / rate[blocks < 1 ? 0 : blocks > 4 ? 3 : blocks - 1];
 }
