@@ -86,3 +86,18 @@ def test_workspace_size_follows_the_plan_without_a_gpu():
     assert ws(256, 256, 9 * 128, _lib.tiled_variant(0, 4)) == 3 * 256 * 256 * 4
     # unsupported shapes need nothing (the GEMM call itself reports the error)
     assert ws(8, 8, 24, _lib.VARIANT_AUTO) == 0
+
+
+def test_grouped_and_blockwise_argument_checks_need_no_gpu():
+    lib = _lib.load()
+    grouped = lib.mi355x_fp8_rowwise_grouped_gemm
+    blockwise = lib.mi355x_fp8_blockwise_gemm
+    # shape and range checks come before anything touches a pointer or a device
+    assert grouped(None, None, None, None, None, None, 0, 64, 64, 64, 64, 64, 64, -1, None) == _lib.EINVAL
+    assert "G must be" in _lib.last_error()
+    assert grouped(None, None, None, None, None, None, 2, 64, 64, 24, 32, 32, 64, -1, None) == _lib.ENOTSUP
+    assert grouped(None, None, None, None, None, None, 2, 64, 64, 64, 64, 64, 64, -1, None) == _lib.EINVAL
+    assert "null" in _lib.last_error()
+    assert blockwise(None, None, None, None, None, 64, 64, 32768 + 128, 40000, 40000, 64, None) == _lib.ENOTSUP
+    assert "K <=" in _lib.last_error()
+    assert blockwise(None, None, None, None, None, 64, 64, 256, 256, 256, 64, None) == _lib.EINVAL
