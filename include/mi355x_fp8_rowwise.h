@@ -109,6 +109,23 @@ int mi355x_fp8_rowwise_gemm(const void* a, const void* b,
                             int variant, void* stream);
 
 /*
+ * The same product with the output element type chosen by the caller: MI355X_FP8_OUT_BF16
+ * (identical to mi355x_fp8_rowwise_gemm) or MI355X_FP8_OUT_F16 (IEEE binary16, round to
+ * nearest even, values beyond 65504 become infinity; `bias` stays bf16). With constant scale
+ * vectors this is the tensor-wise scaled product torch._scaled_mm(a, b, scale_a, scale_b,
+ * out_dtype=float16) computes at tritonbench/operators/fp8_gemm/fp8_gemm.py:87-101.
+ */
+#define MI355X_FP8_OUT_BF16  0
+#define MI355X_FP8_OUT_F16   1
+int mi355x_fp8_rowwise_gemm_ex(const void* a, const void* b,
+                               const float* a_scale, const float* b_scale,
+                               const void* bias, void* c, int out_type,
+                               int64_t M, int64_t N, int64_t K,
+                               int64_t lda, int64_t ldb, int64_t ldc,
+                               void* workspace, size_t workspace_bytes,
+                               int variant, void* stream);
+
+/*
  * Grouped form (mixture-of-experts layers): A and C are G row blocks stacked in one
  * matrix, block g holding m_sizes[g] rows; block g is multiplied with rows
  * [g*N, (g+1)*N) of B:

@@ -73,14 +73,17 @@ def dequant_matmul(
     x_scale: torch.Tensor,
     w_scale: torch.Tensor,
     bias: Optional[torch.Tensor] = None,
+    out_dtype: torch.dtype = torch.bfloat16,
 ) -> torch.Tensor:
-    """The parity reference: fp32 dequantise-then-matmul on host cores, one bf16 rounding."""
+    """The parity reference: fp32 dequantise-then-matmul on host cores, one rounding to the
+    output type (bf16; float16 for the tensor-wise form of
+    tritonbench/operators/fp8_gemm/fp8_gemm.py:87-101)."""
     a = xq.to(torch.float32) * x_scale[:, None]
     b = wq.to(torch.float32) * w_scale[:, None]
     out = a @ b.t()
     if bias is not None:
         out = out + bias.to(torch.float32)
-    return out.to(torch.bfloat16)
+    return out.to(out_dtype)
 
 
 def dequantize(q: torch.Tensor, scale: torch.Tensor) -> torch.Tensor:

@@ -360,3 +360,29 @@ def test_blockwise_operator_cpu_plumbing():
     assert headers == ["(M, N, K)", "torch_cpu_ref-latency", "torch_cpu_ref-tflops"]
     assert table[0][0] == (130, 64, 272)
     assert REGISTERED_BENCHMARKS["fp8_gemm_blockwise"]["_hip_mi355x"].label == "hip_mi355x"
+
+
+def test_tensorwise_operator_cpu_plumbing():
+    from tritonbench_amd.harness.loader import list_operators, load_opbench_by_name
+
+    assert "fp8_gemm" in list_operators()
+    Op = load_opbench_by_name("fp8_gemm")
+    args, extra = get_parser().parse_known_args(
+        ["--op", "fp8_gemm", "--device", "cpu", "--m", "64", "--n", "48", "--k", "32",
+         "--metrics", "latency,tflops,gbps", "--only", "_torch_dequant_cpu"])
+    op = Op(tb_args=args, extra_args=extra)
+    a, b = next(op.get_input_iter())
+    assert a.shape == (64, 32) and b.shape == (32, 48) and b.stride(0) == 1  # b column-major as _scaled_mm wants it
+    out = op._torch_dequant_cpu(a, b)()
+    assert out.dtype == torch.float16
+    op.run(1, 2)
+    headers, table = op.output._table()
+    assert headers == ["(M, N, K)", "torch_cpu_ref-tflops", "torch_cpu_ref-gbps", "torch_cpu_ref-latency"] or \
+        headers == ["(M, N, K)", "torch_cpu_ref-latency", "torch_cpu_ref-tflops", "torch_cpu_ref-gbps"]
+    assert table[0][0] == (64, 48, 32)
+    # default sweep: 2^10 .. 2^14 in quarter steps, square
+    args, extra = get_parser().parse_known_args(["--op", "fp8_gemm", "--device", "cpu"])
+    shapes = Op(tb_args=args, extra_args=extra)._shapes()
+    assert len(shapes) == 20 and shapes[0] == (1024, 1024, 1024) and shapes[1] == (1280, 1280, 1280) and shapes[-1] == (28672, 28672, 28672)
+    args, extra = get_parser().parse_known_args(["--op", "fp8_gemm", "--device", "cpu", "--m", "8", "--n", "8", "--k", "16", "--scaling_rowwise"])
+    assert Op(tb_args=args, extra_args=extra)._torch_dequant_cpu(*next(Op(tb_args=args, extra_args=extra).get_input_iter()))().dtype == torch.bfloat16

@@ -35,6 +35,9 @@ def tiled_variant(config=None, splits=0) -> int:
     return word | ((splits & 0xFF) << 16)
 
 
+OUT_BF16 = 0
+OUT_F16 = 1
+
 SRC_F32 = 0
 SRC_BF16 = 1
 
@@ -47,6 +50,12 @@ SIGNATURES = {
     "mi355x_fp8_rowwise_gemm": (
         c_int,
         [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
+         c_int64, c_int64, c_int64, c_int64, c_int64, c_int64,
+         c_void_p, c_size_t, c_int, c_void_p],
+    ),
+    "mi355x_fp8_rowwise_gemm_ex": (
+        c_int,
+        [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int,
          c_int64, c_int64, c_int64, c_int64, c_int64, c_int64,
          c_void_p, c_size_t, c_int, c_void_p],
     ),

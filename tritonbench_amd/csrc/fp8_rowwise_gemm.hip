@@ -64,6 +64,7 @@ struct GemmParams {
   // (device memory) multiplied with rows [g*N, (g+1)*N) of B and scaled by b_scale[g*N + n]
   const int32_t* m_sizes;
   int groups;
+  int out_f16;  // C holds IEEE binary16 instead of bf16 (same size, same stores)
 };
 
 // Where a tile sits: rows [m0, m_end) of A and C it may touch, first column, group.
@@ -94,6 +95,18 @@ __device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi) {
   uint32_t r;
   asm("v_cvt_pk_bf16_f32 %0, %1, %2" : "=v"(r) : "v"(lo), "v"(hi));
   return r;
+}
+
+// Two f32 -> two IEEE binary16 (round to nearest even; beyond 65504 rounds to infinity as the
+// conversion instruction does); `lo` lands in bits 0..15.
+__device__ __forceinline__ uint32_t pack_f16x2(float lo, float hi) {
+  const _Float16 l = (_Float16)lo, h = (_Float16)hi;
+  return (uint32_t)__builtin_bit_cast(uint16_t, l) | ((uint32_t)__builtin_bit_cast(uint16_t, h) << 16);
+}
+
+// Output element type is a launch parameter (uniform branch, outside the hot loop).
+__device__ __forceinline__ uint32_t pack_out_x2(float lo, float hi, bool f16) {
+  return f16 ? pack_f16x2(lo, hi) : pack_bf16x2(lo, hi);
 }
 
 // ------------------------------------------------------------------------------------
@@ -586,8 +599,14 @@ void gemm_tiled_kernel(GemmParams p) {
 #pragma unroll
           for (int e = 0; e < 8; ++e)
             x[e] = HAS_BIAS ? __builtin_fmaf(x[e], sbv[jp][e], bv[jp][e]) : x[e] * sbv[jp][e];
-          const v4i out = {(int)pack_bf16x2(x[0], x[1]), (int)pack_bf16x2(x[2], x[3]),
-                           (int)pack_bf16x2(x[4], x[5]), (int)pack_bf16x2(x[6], x[7])};
+          v4i out;
+          if (p.out_f16) {
+            out = (v4i){(int)pack_f16x2(x[0], x[1]), (int)pack_f16x2(x[2], x[3]),
+                        (int)pack_f16x2(x[4], x[5]), (int)pack_f16x2(x[6], x[7])};
+          } else {
+            out = (v4i){(int)pack_bf16x2(x[0], x[1]), (int)pack_bf16x2(x[2], x[3]),
+                        (int)pack_bf16x2(x[4], x[5]), (int)pack_bf16x2(x[6], x[7])};
+          }
           const int m = m0 + wm * WTM + i * 32 + r;
           uint16_t* dst = p.c + (size_t)m * p.ldc + n;
           if (ALIGNED) {
@@ -782,7 +801,7 @@ __global__ __launch_bounds__(256) void splitk_finalize_kernel(GemmParams p) {
     const float t = sum[e] * sa_m;
     r[e] = p.bias ? __builtin_fmaf(t, p.b_scale[ne], bf16_to_f32(p.bias[ne])) : t * p.b_scale[ne];
   }
-  const uint32_t lo = pack_bf16x2(r[0], r[1]), hi = pack_bf16x2(r[2], r[3]);
+  const uint32_t lo = pack_out_x2(r[0], r[1], p.out_f16), hi = pack_out_x2(r[2], r[3], p.out_f16);
   uint16_t* dst = p.c + (size_t)m * p.ldc + n;
   if (n + 3 < p.N && ((p.ldc & 3) == 0) && ((reinterpret_cast<uintptr_t>(p.c) & 7) == 0)) {
     *(v2u*)dst = (v2u){lo, hi};
@@ -966,7 +985,7 @@ __global__ __launch_bounds__(KW * 64) void gemm_skinny_kernel(GemmParams p) {
       r[e] = sum[e] * fin_sa * fin_sb[e];
       if (p.bias) r[e] += fin_bias[e];
     }
-    const uint32_t lo = pack_bf16x2(r[0], r[1]), hi = pack_bf16x2(r[2], r[3]);
+    const uint32_t lo = pack_out_x2(r[0], r[1], p.out_f16), hi = pack_out_x2(r[2], r[3], p.out_f16);
     uint16_t* dst = p.c + (size_t)fin_m * p.ldc + fin_n;
     if (fin_n + 3 < p.N && ((p.ldc & 3) == 0) && ((reinterpret_cast<uintptr_t>(p.c) & 7) == 0)) {
       *(v2u*)dst = (v2u){lo, hi};
@@ -1387,6 +1406,16 @@ int mi355x_fp8_rowwise_gemm(const void* a, const void* b, const float* a_scale, 
                             const void* bias, void* c, int64_t M, int64_t N, int64_t K, int64_t lda,
                             int64_t ldb, int64_t ldc, void* workspace, size_t workspace_bytes,
                             int variant, void* stream) {
+  return mi355x_fp8_rowwise_gemm_ex(a, b, a_scale, b_scale, bias, c, MI355X_FP8_OUT_BF16, M, N, K, lda, ldb, ldc,
+                                    workspace, workspace_bytes, variant, stream);
+}
+
+int mi355x_fp8_rowwise_gemm_ex(const void* a, const void* b, const float* a_scale, const float* b_scale,
+                               const void* bias, void* c, int out_type, int64_t M, int64_t N, int64_t K,
+                               int64_t lda, int64_t ldb, int64_t ldc, void* workspace, size_t workspace_bytes,
+                               int variant, void* stream) {
+  if (out_type != MI355X_FP8_OUT_BF16 && out_type != MI355X_FP8_OUT_F16)
+    return fail(MI355X_FP8_EINVAL, "unknown output type %d", out_type);
   int st = check_shape(M, N, K);
   if (st != MI355X_FP8_OK) return st;
   if (!a || !b || !a_scale || !b_scale || !c) return fail(MI355X_FP8_EINVAL, "null operand pointer");
@@ -1425,7 +1454,7 @@ int mi355x_fp8_rowwise_gemm(const void* a, const void* b, const float* a_scale, 
   p.lda = lda; p.ldb = ldb; p.ldc = ldc;
   p.tiles_m = p.tiles_n = 0; p.group_m = 1;
   p.splits = 1; p.steps_per_split = k_steps_of(K); p.partial = nullptr;
-  p.m_sizes = nullptr; p.groups = 0;
+  p.m_sizes = nullptr; p.groups = 0; p.out_f16 = out_type == MI355X_FP8_OUT_F16;
   hipStream_t s = (hipStream_t)stream;
 
   switch (variant) {
@@ -1500,7 +1529,7 @@ int mi355x_fp8_rowwise_grouped_gemm(const void* a, const void* b, const float* a
   p.lda = lda; p.ldb = ldb; p.ldc = ldc;
   p.tiles_m = p.tiles_n = 0; p.group_m = 1;
   p.splits = 1; p.steps_per_split = k_steps_of(K); p.partial = nullptr;
-  p.m_sizes = m_sizes; p.groups = (int)G;
+  p.m_sizes = m_sizes; p.groups = (int)G; p.out_f16 = 0;
   hipStream_t s = (hipStream_t)stream;
   // Large tiles when an average group fills most of one and there are enough of them for every
   // CU, small tiles otherwise (the group sizes themselves are on the device; M / G is what the
@@ -1542,7 +1571,7 @@ int mi355x_fp8_blockwise_gemm(const void* a, const void* b, const float* a_scale
   p.lda = lda; p.ldb = ldb; p.ldc = ldc;
   p.tiles_m = p.tiles_n = 0; p.group_m = 1;
   p.splits = 1; p.steps_per_split = k_steps_of(K); p.partial = nullptr;
-  p.m_sizes = nullptr; p.groups = 0;
+  p.m_sizes = nullptr; p.groups = 0; p.out_f16 = 0;
   hipStream_t s = (hipStream_t)stream;
   // 128x128 tiles: with 256x128 tiles (64 more accumulators and 64 more partial products per
   // lane) the fold no longer fits the 256 registers VALU instructions can address

@@ -1,6 +1,6 @@
 """PyTorch-facing wrappers around the C ABI. PyTorch supplies device memory and the
 current stream; all arithmetic happens in the HIP library."""
-from typing import Optional, Tuple
+from typing import Callable, Optional, Tuple
 
 import torch
 
@@ -45,8 +45,10 @@ def fp8_gemm_rowwise(
     out: Optional[torch.Tensor] = None,
     variant: int = _lib.VARIANT_AUTO,
     workspace: Optional[torch.Tensor] = None,
+    out_dtype: torch.dtype = torch.bfloat16,
 ) -> torch.Tensor:
-    """bf16 [M,N] = ((xq @ wq.T) * x_scale[:,None] * w_scale[None,:] + bias).
+    """[M,N] = ((xq @ wq.T) * x_scale[:,None] * w_scale[None,:] + bias) in bfloat16 (default)
+    or float16 (`out_dtype`).
 
     Same operands as the callables of tritonbench/operators/fp8_gemm_rowwise/operator.py:187-217:
     xq [M,K] and wq [N,K] float8_e4m3fn, x_scale [M] and w_scale [N] float32, bias [N]
@@ -78,12 +80,14 @@ def fp8_gemm_rowwise(
         if bias.dtype != torch.bfloat16 or bias.numel() != n or not bias.is_contiguous():
             raise ValueError("bias must be a contiguous bfloat16 vector of N entries")
         bias_ptr = bias.data_ptr()
+    if out_dtype not in (torch.bfloat16, torch.float16):
+        raise TypeError(f"out_dtype must be bfloat16 or float16, got {out_dtype}")
     if out is None:
-        out = torch.empty((m, n), dtype=torch.bfloat16, device=xq.device)
+        out = torch.empty((m, n), dtype=out_dtype, device=xq.device)
     else:
         _require_gpu(out, "out")
-        if out.dtype != torch.bfloat16 or tuple(out.shape) != (m, n) or out.stride(1) != 1:
-            raise ValueError("out must be bfloat16 [M,N] with unit column stride")
+        if out.dtype != out_dtype or tuple(out.shape) != (m, n) or out.stride(1) != 1:
+            raise ValueError(f"out must be {out_dtype} [M,N] with unit column stride")
     if workspace is not None:
         _require_gpu(workspace, "workspace")
         if not workspace.is_contiguous():
@@ -92,13 +96,40 @@ def fp8_gemm_rowwise(
     else:
         ws_bytes = lib.mi355x_fp8_rowwise_workspace_bytes(m, n, k, variant)
         ws = torch.empty(ws_bytes, dtype=torch.uint8, device=xq.device) if ws_bytes else None
-    st = lib.mi355x_fp8_rowwise_gemm(
+    st = lib.mi355x_fp8_rowwise_gemm_ex(
         xq.data_ptr(), wq.data_ptr(), x_scale.data_ptr(), w_scale.data_ptr(), bias_ptr,
-        out.data_ptr(), m, n, k, xq.stride(0), wq.stride(0), out.stride(0),
+        out.data_ptr(), _lib.OUT_F16 if out_dtype == torch.float16 else _lib.OUT_BF16,
+        m, n, k, xq.stride(0), wq.stride(0), out.stride(0),
         ws.data_ptr() if ws is not None else None, ws_bytes, variant, _stream_ptr(),
     )
     _lib.check(st, "mi355x_fp8_rowwise_gemm")
     return out
+
+
+def fp8_gemm_tensorwise(
+    a: torch.Tensor,
+    b: torch.Tensor,
+    scale_a: torch.Tensor,
+    scale_b: torch.Tensor,
+    out_dtype: torch.dtype = torch.float16,
+    out: Optional[torch.Tensor] = None,
+) -> Callable[[], torch.Tensor]:
+    """Tensor-wise scaled product with the operands of torch._scaled_mm as the reference's
+    fp8_gemm operator passes them (tritonbench/operators/fp8_gemm/fp8_gemm.py:57-101):
+    a [M,K] row-major, b [K,N] column-major (b.T is [N,K] K-contiguous), scale_a and scale_b
+    one-element float32 DEVICE tensors (or [M,1] / [1,N] for its row-wise flag). Returns a
+    zero-argument callable; the scalars are spread into vectors on the device here, once,
+    outside the callable, and never read by the host."""
+    if b.dim() != 2 or b.stride(0) != 1:
+        raise ValueError("b must be [K,N] column-major (b.T contiguous), as torch._scaled_mm wants it")
+    m, n = a.shape[0], b.shape[1]
+    xs = scale_a.to(torch.float32).reshape(-1).expand(m).contiguous() if scale_a.numel() == 1 else scale_a.reshape(-1).contiguous()
+    ws = scale_b.to(torch.float32).reshape(-1).expand(n).contiguous() if scale_b.numel() == 1 else scale_b.reshape(-1).contiguous()
+    wq = b.t()
+    if out is None:
+        out = torch.empty((m, n), dtype=out_dtype, device=a.device)
+    space = gemm_workspace(m, n, a.shape[1], a.device)
+    return lambda: fp8_gemm_rowwise(a, wq, xs, ws, out=out, workspace=space, out_dtype=out_dtype)
 
 
 def fp8_gemm_rowwise_grouped(
