@@ -386,3 +386,26 @@ def test_tensorwise_operator_cpu_plumbing():
     assert len(shapes) == 20 and shapes[0] == (1024, 1024, 1024) and shapes[1] == (1280, 1280, 1280) and shapes[-1] == (28672, 28672, 28672)
     args, extra = get_parser().parse_known_args(["--op", "fp8_gemm", "--device", "cpu", "--m", "8", "--n", "8", "--k", "16", "--scaling_rowwise"])
     assert Op(tb_args=args, extra_args=extra)._torch_dequant_cpu(*next(Op(tb_args=args, extra_args=extra).get_input_iter()))().dtype == torch.bfloat16
+
+
+def test_export_dumps_inputs_and_outputs(tmp_path):
+    from tritonbench_amd.harness.loader import load_opbench_by_name
+
+    Op = load_opbench_by_name("fp8_gemm_rowwise")
+    args, extra = get_parser().parse_known_args(
+        ["--op", "fp8_gemm_rowwise", "--device", "cpu", "--m", "32", "--n", "48", "--k", "64", "--metrics", "latency",
+         "--only", "_torch_dequant_cpu", "--export", "both", "--export-dir", str(tmp_path)])
+    op = Op(tb_args=args, extra_args=extra)
+    op.run(1, 1)
+    files = sorted(f.name for f in tmp_path.iterdir())
+    assert files == ["x_(32,48,64)-_torch_dequant_cpu-fwd-output.pt", "x_(32,48,64)-input.pt"]
+    xq, wq, xs, ws, bias = torch.load(tmp_path / "x_(32,48,64)-input.pt", weights_only=True)
+    out = torch.load(tmp_path / "x_(32,48,64)-_torch_dequant_cpu-fwd-output.pt", weights_only=True)
+    assert xq.dtype == torch.float8_e4m3fn and xq.shape == (32, 64) and bias is None and out.shape == (32, 48)
+    from oracle import fp8_rowwise as orc
+    assert torch.equal(out, orc.dequant_matmul(xq, wq, xs, ws))
+    args, extra = get_parser().parse_known_args(
+        ["--op", "fp8_gemm_rowwise", "--device", "cpu", "--m", "32", "--n", "48", "--k", "64", "--only", "_torch_dequant_cpu",
+         "--export", "input", "--export-dir", str(tmp_path / "missing")])
+    with pytest.raises(RuntimeError, match="must exist"):
+        Op(tb_args=args, extra_args=extra).run(1, 1)

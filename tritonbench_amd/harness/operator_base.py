@@ -368,6 +368,11 @@ class BenchmarkOperator(metaclass=_PostInit):
             fn = self._get_bm_func(fn_name)
             if baseline:
                 self.baseline_fn = fn
+            if getattr(self.tb_args, "export", None) in ("output", "both"):
+                from .export import export_output
+
+                export_output(self.get_x_val(self.example_inputs), fn_name, self.mode.value, fn,
+                              getattr(self.tb_args, "export_dir", None))
             backend_device = getattr(fn, "device", self.device)
             if want & {"latency", "tflops", "speedup", "gbps"} or any(m in want for m in R.REGISTERED_METRICS.get(self.name, [])):
                 rec.latency = do_bench_wrapper(
@@ -417,6 +422,10 @@ class BenchmarkOperator(metaclass=_PostInit):
                     break
                 self.example_inputs = input_cast(lambda x: isinstance(x, torch.Tensor), lambda x: x.to(self.device), ex)
                 x_val = self.get_x_val(self.example_inputs)
+                if getattr(self.tb_args, "export", None) in ("input", "both"):
+                    from .export import export_input
+
+                    export_input(x_val, self.example_inputs, getattr(self.tb_args, "export_dir", None))
                 self.baseline_fn = None
                 self.baseline_metrics = None
                 per_backend: Dict[str, BenchmarkOperatorMetrics] = {}

@@ -31,5 +31,8 @@ def get_parser() -> argparse.ArgumentParser:
     p.add_argument("--test-only", action="store_true", help="run each backend once, no timing loops")
     p.add_argument("--rtol", type=float, default=None)
     p.add_argument("--atol", type=float, default=None)
+    p.add_argument("--export", choices=["input", "output", "both"], default=None,
+                   help="dump the inputs and/or every backend's output as .pt files")
+    p.add_argument("--export-dir", default=None, help="existing directory for --export")
     p.add_argument("--list-backends", action="store_true")
     return p
