@@ -925,12 +925,37 @@ __global__ __launch_bounds__(KW * 64) void gemm_skinny_kernel(GemmParams p) {
   };
 
   // The loop is unrolled DEPTH times so every register set has a fixed name; the compiler's
-  // own wait counts make each consume() wait for exactly its set's loads (they return in
-  // issue order, so the younger sets stay in flight).
+  // own wait counts then make each consume() wait for exactly its set's loads (they return
+  // in issue order, so the younger sets stay in flight). That only works on paths without
+  // conditional fetches: where paths with different numbers of younger loads meet, the
+  // compiler has to assume the fewest and ends up draining the whole queue once per round.
+  // So the rounds in which every consume is followed by a fetch form their own loop, the
+  // last full round (consumes only) is straight-line code, and only ragged step counts take
+  // the conditional form. (Measured: worth 2 % with four steps in flight; with two steps in
+  // flight the drained form is 8-11 % faster, so those configurations keep it.)
+  constexpr bool kSteadyLoop = DEPTH >= 4;
+  int i = 0;
+  if (kSteadyLoop && my_steps >= DEPTH) {
 #pragma unroll
-  for (int d = 0; d < DEPTH; ++d)
-    if (d < my_steps) fetch(d, land[d]);
-  for (int i = 0; i < my_steps; i += DEPTH) {
+    for (int d = 0; d < DEPTH; ++d) fetch(d, land[d]);
+    for (; i + 2 * DEPTH <= my_steps; i += DEPTH) {
+#pragma unroll
+      for (int d = 0; d < DEPTH; ++d) {
+        consume(land[d]);
+        fetch(i + d + DEPTH, land[d]);
+      }
+    }
+    if (i + DEPTH == my_steps) {
+#pragma unroll
+      for (int d = 0; d < DEPTH; ++d) consume(land[d]);
+      i += DEPTH;
+    }
+  } else {
+#pragma unroll
+    for (int d = 0; d < DEPTH; ++d)
+      if (d < my_steps) fetch(d, land[d]);
+  }
+  for (; i < my_steps; i += DEPTH) {
 #pragma unroll
     for (int d = 0; d < DEPTH; ++d) {
       if (i + d < my_steps) {
