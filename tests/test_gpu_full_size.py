@@ -109,3 +109,17 @@ def test_c4_llama70b_projections(gpu_device, name):
         rows = torch.arange(m) if m <= 32 else _sample_rows(m, 24 if n > 20000 else 48)
         _check_rows(out, xq, wq, xs, ws, None, rows, sigma, b_deq)
         del out, dxq, dxs
+
+
+def test_output_beyond_2_to_31_elements(gpu_device):
+    # 32800 x 65600 bf16 = 2.15e9 elements (4.3 GB): row offsets into C pass both 2^31 elements
+    # and 2^32 bytes; K is one step, so the case costs a few hundred microseconds of GPU time
+    m, n, k = 32800, 65600, 128
+    xq, wq, xs, ws, b = orc.make_inputs(m, n, k, 1.0, True)
+    dxq, dwq, dxs, dws, db = _gpu(gpu_device, xq, wq, xs, ws, b)
+    out = ops.fp8_gemm_rowwise(dxq, dwq, dxs, dws, bias=db)
+    torch.cuda.synchronize()
+    first_past = 2 ** 31 // n  # the row whose elements straddle index 2^31
+    rows = sorted({0, 1, m - 1, m - 2, first_past - 1, first_past, first_past + 1, 2 ** 32 // (2 * n), m // 2, 12345})
+    _check_rows(out, xq, wq, xs, ws, b, torch.tensor(rows, dtype=torch.long), 1.0)
+    del out

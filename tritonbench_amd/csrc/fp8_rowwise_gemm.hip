@@ -783,17 +783,26 @@ __global__ __launch_bounds__(256) void splitk_finalize_kernel(GemmParams p) {
   const size_t plane = (size_t)p.M * p.N;
   const float* src = p.partial + (size_t)m * p.N + n;
   const bool vec = (p.N & 3) == 0;  // then n + 3 < N and every row start is 16-byte aligned
+  const float sa_m = p.a_scale[m];  // fetched beside the partial sums, not after them
   v4f sum = {0.f, 0.f, 0.f, 0.f};
-  for (int s = 0; s < p.splits; ++s) {
-    if (vec) {
-      sum += *(const v4f*)(src + s * plane);
-    } else {
+  if (vec) {
+    // four splits' loads in flight at a time; added in split order, as the scalar form does
+    int s = 0;
+    for (; s + 4 <= p.splits; s += 4) {
+      v4f part[4];
+#pragma unroll
+      for (int u = 0; u < 4; ++u) part[u] = __builtin_nontemporal_load((const v4f*)(src + (s + u) * plane));
+#pragma unroll
+      for (int u = 0; u < 4; ++u) sum += part[u];
+    }
+    for (; s < p.splits; ++s) sum += __builtin_nontemporal_load((const v4f*)(src + s * plane));
+  } else {
+    for (int s = 0; s < p.splits; ++s) {
 #pragma unroll
       for (int e = 0; e < 4; ++e)
         if (n + e < p.N) sum[e] += src[s * plane + e];
     }
   }
-  const float sa_m = p.a_scale[m];
   float r[4];
 #pragma unroll
   for (int e = 0; e < 4; ++e) {
