@@ -334,32 +334,65 @@ void gemm_tiled_kernel(GemmParams p) {
   StepCursor ca = {walk.slot, 0, 0, 0}, cb = {walk.slot, 0, 0, 0};
   const uint8_t* l_a = nullptr;
   const uint8_t* l_b = nullptr;
-  uint32_t a_off[A_GROUPS], b_off[B_GROUPS];
-  // Rows past the matrix edge are redirected to the last valid row: they are read but never
-  // stored, so every load stays in bounds without predication.
+  // Source address of a lane's 16 bytes in the i-th 8-row group (grp = wave + NW*i) a wave fetches:
+  // tile base + K offset + a 32-bit lane offset, row*ld + chunk, with rows past the matrix edge
+  // redirected to the last valid row (they are read but never stored, so every load stays in
+  // bounds without predication). Two forms:
+  //  * one offset register per group (small tiles);
+  //  * 256x256 tile, where registers are short (16 of these per lane used to end up in scratch,
+  //    and every reload there waits for all loads in flight): 8*grp*ld goes into the scalar
+  //    base and the lane part, ld_row*ld + chunk, is one register for all groups (the chunk
+  //    depends on the group's parity only, which a wave's groups share). Only the group that
+  //    holds the edge needs its own lane part (rows clamped inside the group); groups behind it
+  //    are sent there too. Costs a few scalar instructions and a select per load.
+  static_assert(NW % 2 == 0, "all groups of a wave must share their parity");
+  constexpr bool SHARED_OFFSETS = BM * BN >= 256 * 256;
+  constexpr int MAX_GROUPS = A_GROUPS > B_GROUPS ? A_GROUPS : B_GROUPS;
+  struct OperandOffsets {
+    uint32_t per_group[SHARED_OFFSETS ? 1 : MAX_GROUPS];
+    uint32_t full, edge;  // shared form: lane part of whole groups / of the group with the edge
+    int last_group;       // shared form: the group that holds the last valid row
+    uint32_t ld;
+  };
+  // 24-bit multiplies (row < 2^8, leading dimension < 2^24 by the host's check): one instruction
+  // and a 32-bit result, where the full multiply leaves a 64-bit register pair
+  auto make_offsets = [&](int rows_valid, long ld, int groups) -> OperandOffsets {
+    const int last_row = max(rows_valid - 1, 0);
+    OperandOffsets o = {{0}, 0, 0, 0, (uint32_t)ld};
+    if (SHARED_OFFSETS) {
+      const uint32_t chunk = ld_chunk_off(wave);
+      o.full = __umul24((uint32_t)ld_row, (uint32_t)ld) + chunk;
+      o.edge = __umul24((uint32_t)min(ld_row, last_row & 7), (uint32_t)ld) + chunk;
+      o.last_group = last_row >> 3;
+    } else {
+#pragma unroll
+      for (int i = 0; i < MAX_GROUPS; ++i) {
+        const int grp = wave + NW * i;
+        if (i < groups) o.per_group[i] = __umul24((uint32_t)min(grp * 8 + ld_row, last_row), (uint32_t)ld) + ld_chunk_off(grp);
+      }
+    }
+    return o;
+  };
+  auto group_src = [&](const uint8_t* g, const OperandOffsets& o, int i) -> const uint8_t* {
+    if (!SHARED_OFFSETS) return g + o.per_group[i];
+    const int grp = wave + NW * i;
+    const uint32_t rows_off = (uint32_t)min(grp, o.last_group) * 8u * o.ld;  // < 2^32 by the same check
+    return g + rows_off + (grp < o.last_group ? o.full : o.edge);
+  };
+  OperandOffsets a_off = {{0}, 0, 0, 0, 0}, b_off = {{0}, 0, 0, 0, 0};
   auto setup_a = [&](int li) {
     const TileLoc loc = locate(walk_a, li);
     ca.kt = split_begin(item_split(li));
     ca.kt_end = split_end(item_split(li));
-    const int m0 = loc.m0;
-    l_a = p.a + (size_t)m0 * p.lda;
-#pragma unroll
-    for (int i = 0; i < A_GROUPS; ++i) {
-      const int grp = wave + NW * i;
-      a_off[i] = (uint32_t)min(grp * 8 + ld_row, loc.m_end - 1 - m0) * (uint32_t)p.lda + ld_chunk_off(grp);
-    }
+    l_a = p.a + (size_t)loc.m0 * p.lda;
+    a_off = make_offsets(loc.m_end - loc.m0, p.lda, A_GROUPS);
   };
   auto setup_b = [&](int li) {
     const TileLoc loc = locate(walk_b, li);
     cb.kt = split_begin(item_split(li));
     cb.kt_end = split_end(item_split(li));
-    const int n0 = loc.n0;
-    l_b = p.b + ((size_t)loc.group * p.N + n0) * p.ldb;
-#pragma unroll
-    for (int i = 0; i < B_GROUPS; ++i) {
-      const int grp = wave + NW * i;
-      b_off[i] = (uint32_t)min(grp * 8 + ld_row, p.N - 1 - n0) * (uint32_t)p.ldb + ld_chunk_off(grp);
-    }
+    l_b = p.b + ((size_t)loc.group * p.N + loc.n0) * p.ldb;
+    b_off = make_offsets(p.N - loc.n0, p.ldb, B_GROUPS);
   };
   // Issues one operand's loads for its cursor's step into stage (issued % STAGES). Past the
   // last step it re-issues the last one into a stage nobody reads again, which keeps the
@@ -367,19 +400,17 @@ void gemm_tiled_kernel(GemmParams p) {
   // K tail (KTAIL kernels only): in the partial last step, lanes whose chunk lies at or past
   // K fetch the zero chunk instead. A lane's logical chunk is the same for all its groups
   // (the swizzle key depends on the group's parity only, and a wave's groups are NW apart).
-  static_assert(NW % 2 == 0, "all groups of a wave must share their parity");
   const bool tail_chunk_ok = ((ld_pc ^ swz128(wave * 8 + ld_row)) * kChunk) < k_tail;
-  auto chunk_src = [&](const uint8_t* g, uint32_t off, bool real) -> const uint8_t* {
-    if (!KTAIL) return g + off;
-    return real ? g + off : reinterpret_cast<const uint8_t*>(&kZeroChunk);
+  auto chunk_src = [&](const uint8_t* g, const OperandOffsets& o, int i, bool real) -> const uint8_t* {
+    if (!KTAIL) return group_src(g, o, i);
+    return real ? group_src(g, o, i) : reinterpret_cast<const uint8_t*>(&kZeroChunk);
   };
-  constexpr int MAX_GROUPS = A_GROUPS > B_GROUPS ? A_GROUPS : B_GROUPS;
-  auto issue = [&](const uint8_t* gbase, const uint32_t* off, int groups, int kt, uint8_t* sbase) {
+  auto issue = [&](const uint8_t* gbase, const OperandOffsets& off, int groups, int kt, uint8_t* sbase) {
     const uint8_t* g = gbase + (size_t)kt * kStepK;
     const bool real = !KTAIL || kt < k_full || tail_chunk_ok;
 #pragma unroll
     for (int i = 0; i < MAX_GROUPS; ++i)
-      if (i < groups) load_chunk_to_lds(chunk_src(g, off[i], real), sbase + (wave + NW * i) * 1024);
+      if (i < groups) load_chunk_to_lds(chunk_src(g, off, i, real), sbase + (wave + NW * i) * 1024);
   };
   auto issue_a = [&]() {
     issue(l_a, a_off, A_GROUPS, ca.kt, lds + (ca.issued % kStagesA) * STAGE_A);
@@ -527,7 +558,8 @@ void gemm_tiled_kernel(GemmParams p) {
     // The lane-dependent addresses below are the same for every tile; derived from an opaque
     // copy of the lane id they are recomputed here (a few integer operations) instead of
     // being hoisted out of the tile loop, where they would occupy registers through the K loop.
-    int lane_e = lane;
+    // (the lane id itself comes from the hardware's lane count, so not even it stays live)
+    int lane_e = (int)__builtin_amdgcn_mbcnt_hi(~0u, __builtin_amdgcn_mbcnt_lo(~0u, 0u));
     asm volatile("" : "+v"(lane_e));
     const int l32 = lane_e & 31, half = lane_e >> 5;
     uint8_t* const wr_row = row_addr(l32);
@@ -685,7 +717,7 @@ void gemm_tiled_kernel(GemmParams p) {
         mfma_one(xa, xb, t, BLOCKSCALE || FIRST);
 #pragma unroll
         for (int l = 0; l < B_GROUPS; ++l)
-          if (l * NMFMA / B_GROUPS == t) load_chunk_to_lds(chunk_src(gb, b_off[l], real), wb + NW * l * 1024);
+          if (l * NMFMA / B_GROUPS == t) load_chunk_to_lds(chunk_src(gb, b_off, l, real), wb + NW * l * 1024);
 #pragma unroll
         for (int u = t * RPS; u < (t + 1) * RPS; ++u)
           if (u < NREAD) read_one(ya, yb, cur_a, cur_b, 1, u);
@@ -713,7 +745,7 @@ void gemm_tiled_kernel(GemmParams p) {
         mfma_one(ya, yb, t, false);
 #pragma unroll
         for (int l = 0; l < A_GROUPS; ++l)
-          if (l * NMFMA / A_GROUPS == t) load_chunk_to_lds(chunk_src(ga, a_off[l], real), wa + NW * l * 1024);
+          if (l * NMFMA / A_GROUPS == t) load_chunk_to_lds(chunk_src(ga, a_off, l, real), wa + NW * l * 1024);
 #pragma unroll
         for (int u = t * RPS; u < (t + 1) * RPS; ++u)
           if (READ_NEXT && u < NREAD) read_one(xa, xb, nxt_a, nxt_b, 0, u);
