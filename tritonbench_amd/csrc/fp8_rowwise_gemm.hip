@@ -642,7 +642,7 @@ void gemm_tiled_kernel(GemmParams p) {
           const int m = m0 + wm * WTM + i * 32 + r;
           uint16_t* dst = p.c + (size_t)m * p.ldc + n;
           if (ALIGNED) {
-            *(v4i*)dst = out;
+            __builtin_nontemporal_store(out, (v4i*)dst);  // written once, read by a later kernel at best
           } else if (m < loc.m_end) {
 #pragma unroll
             for (int e = 0; e < 8; ++e)
