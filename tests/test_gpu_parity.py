@@ -309,10 +309,14 @@ def test_unsupported_and_invalid_arguments_raise(gpu_device):
 
 def test_dispatch_is_pinned(gpu_device):
     assert ops.select_variant(16, 8192, 8192) == _lib.VARIANT_SKINNY
-    assert ops.select_variant(64, 8192, 8192) == _lib.VARIANT_SKINNY
+    assert ops.select_variant(32, 2048, 2048) == _lib.VARIANT_SKINNY
     assert ops.select_variant(8192, 8192, 8192) == _lib.VARIANT_TILED
-    # M <= 64 with a long weight panel and four 16-row blocks of A: 64-row tiles win
+    # three or four 16-row blocks of A, or two with a long weight panel: split-K tiles that
+    # fetch B with the streaming policy win
+    assert ops.select_variant(64, 8192, 8192) == _lib.VARIANT_TILED
+    assert ops.select_variant(48, 10240, 8192) == _lib.VARIANT_TILED
     assert ops.select_variant(64, 57344, 8192) == _lib.VARIANT_TILED
+    assert ops.select_variant(32, 57344, 8192) == _lib.VARIANT_TILED
     assert ops.select_variant(16, 57344, 8192) == _lib.VARIANT_SKINNY
 
 

@@ -159,11 +159,14 @@ constexpr int kDefaultDist = 2;  // steps a load runs ahead of its use; A ring =
 
 __device__ __forceinline__ int swz128(int row) { return (row >> 1) & 7; }
 
+// STREAM marks the lines as used once (the instruction's `nt` bit): they leave the L2 early
+// instead of pushing out lines other workgroups will ask for again.
+template <bool STREAM = false>
 __device__ __forceinline__ void load_chunk_to_lds(const uint8_t* gsrc, uint8_t* lds_wave_base) {
   // Each lane fetches 16 bytes; the hardware deposits lane i's bytes at lds_wave_base + 16*i.
   __builtin_amdgcn_global_load_lds(
       (const __attribute__((address_space(1))) void*)gsrc,
-      (__attribute__((address_space(3))) void*)lds_wave_base, 16, 0, 0);
+      (__attribute__((address_space(3))) void*)lds_wave_base, 16, 0, STREAM ? 2 : 0);
 }
 
 // Source of the chunks that lie past K in the last, partial K step: the operands there must
@@ -185,7 +188,7 @@ __device__ __forceinline__ void wait_loads_and_barrier() {
 // Cursor over the (tile, K step) sequence a workgroup walks; one for the A loads, one for
 // the B loads (which run a step further ahead).
 struct StepCursor {
-  int item, kt, kt_end, issued;
+  int item, kt, kt_begin, kt_end, left, issued;  // kt walks [kt_begin, kt_end) cyclically, `left` steps to go
 };
 
 // The kernel is one software pipeline over "steps" (a 128-byte K slab of one tile) that runs
@@ -224,8 +227,13 @@ constexpr int tiled_wgs_per_cu(int BM, int BN, bool blockscale = false, int dist
 // inside one scale block and 128-byte steps that factor is one number per wave and step:
 // the MFMAs of a step go to a second accumulator set, which is folded into the first
 // (acc += s * tmp) behind the next step's MFMAs.
+//
+// STREAM_B: the rows of B are fetched with the streaming cache policy. For launches with one or
+// two tile rows, where a panel of B is read by one or two workgroups and never again
+// (measured: M=128, N=K=8192 27.6 -> 24.2 us, M=64 22.5 -> 19.6 us; with more tile rows the
+// panels are shared through the L2 and the same policy costs 5-8 %).
 template <int BM, int BN, int WAVES_M, int WAVES_N, bool KTAIL, int EPI, bool GROUPED = false, bool BLOCKSCALE = false,
-          int DIST = kDefaultDist>
+          int DIST = kDefaultDist, bool STREAM_B = false>
 __global__ __launch_bounds__(WAVES_M* WAVES_N * 64)
 __attribute__((amdgpu_waves_per_eu(tiled_wgs_per_cu(BM, BN, BLOCKSCALE, DIST) * WAVES_M * WAVES_N / 4,
                                    tiled_wgs_per_cu(BM, BN, BLOCKSCALE, DIST) * WAVES_M * WAVES_N / 4)))
@@ -233,6 +241,7 @@ void gemm_tiled_kernel(GemmParams p) {
   constexpr int kStagesA = DIST, kStagesB = DIST + 1;
   static_assert(DIST >= 2 && tiled_lds_bytes(BM, BN, DIST) <= 160 * 1024, "the stage rings must fit the LDS");
   static_assert(!GROUPED || EPI == kEpiPlain, "the grouped form has neither bias nor split-K");
+  static_assert(!STREAM_B || (!BLOCKSCALE && !GROUPED), "the rotated K order is for the plain form only");
   static_assert(!BLOCKSCALE || (128 % (BM / WAVES_M) == 0 && 128 % (BN / WAVES_N) == 0 && EPI == kEpiPlain && !GROUPED),
                 "a wave's tile must lie inside one 128x128 scale block: one factor per wave and step");
   constexpr bool HAS_BIAS = EPI == kEpiBias;
@@ -331,7 +340,21 @@ void gemm_tiled_kernel(GemmParams p) {
   GroupWalk walk_a = first_group(), walk_b = first_group(), walk_c = first_group();
 
   // ---- load side of the pipeline
-  StepCursor ca = {walk.slot, 0, 0, 0}, cb = {walk.slot, 0, 0, 0};
+  StepCursor ca = {walk.slot, 0, 0, 0, 0, 0}, cb = {walk.slot, 0, 0, 0, 0, 0};
+  // STREAM_B launches start every tile column at a different K step and wrap around. Their
+  // workgroups stream disjoint rows of B in lockstep; with a power-of-two row pitch all the
+  // addresses in flight at one moment would agree in their low bits and crowd a few memory
+  // channels (M=32, N=57344, K=8192 with an 8192-byte pitch: 100 us; the same data at a pitch
+  // of 8320 bytes: 71 us). The sum over K does not care where it starts. Launches whose tiles
+  // share panels of B through the L2 keep the common order: there the sharing needs it. So do
+  // plans with more than two splits, whose items are already spread over K (M=128, N=K=8192 with
+  // four splits lost 5 % to the rotation; two splits gain 5 %, unsplit plans 11-28 %).
+  auto start_cursor = [&](StepCursor& c, int li, const TileLoc& loc) {
+    c.kt_begin = split_begin(item_split(li));
+    c.kt_end = split_end(item_split(li));
+    c.left = c.kt_end - c.kt_begin;
+    c.kt = c.kt_begin + (STREAM_B && p.splits <= 2 ? (loc.n0 / BN) % c.left : 0);
+  };
   const uint8_t* l_a = nullptr;
   const uint8_t* l_b = nullptr;
   // Source address of a lane's 16 bytes in the i-th 8-row group (grp = wave + NW*i) a wave fetches:
@@ -382,15 +405,13 @@ void gemm_tiled_kernel(GemmParams p) {
   OperandOffsets a_off = {{0}, 0, 0, 0, 0}, b_off = {{0}, 0, 0, 0, 0};
   auto setup_a = [&](int li) {
     const TileLoc loc = locate(walk_a, li);
-    ca.kt = split_begin(item_split(li));
-    ca.kt_end = split_end(item_split(li));
+    start_cursor(ca, li, loc);
     l_a = p.a + (size_t)loc.m0 * p.lda;
     a_off = make_offsets(loc.m_end - loc.m0, p.lda, A_GROUPS);
   };
   auto setup_b = [&](int li) {
     const TileLoc loc = locate(walk_b, li);
-    cb.kt = split_begin(item_split(li));
-    cb.kt_end = split_end(item_split(li));
+    start_cursor(cb, li, loc);
     l_b = p.b + ((size_t)loc.group * p.N + loc.n0) * p.ldb;
     b_off = make_offsets(p.N - loc.n0, p.ldb, B_GROUPS);
   };
@@ -405,33 +426,39 @@ void gemm_tiled_kernel(GemmParams p) {
     if (!KTAIL) return group_src(g, o, i);
     return real ? group_src(g, o, i) : reinterpret_cast<const uint8_t*>(&kZeroChunk);
   };
-  auto issue = [&](const uint8_t* gbase, const OperandOffsets& off, int groups, int kt, uint8_t* sbase) {
+  auto issue = [&](auto stream_tag, const uint8_t* gbase, const OperandOffsets& off, int groups, int kt, uint8_t* sbase) {
     const uint8_t* g = gbase + (size_t)kt * kStepK;
     const bool real = !KTAIL || kt < k_full || tail_chunk_ok;
 #pragma unroll
     for (int i = 0; i < MAX_GROUPS; ++i)
-      if (i < groups) load_chunk_to_lds(chunk_src(g, off, i, real), sbase + (wave + NW * i) * 1024);
+      if (i < groups)
+        load_chunk_to_lds<decltype(stream_tag)::value>(chunk_src(g, off, i, real), sbase + (wave + NW * i) * 1024);
   };
   auto issue_a = [&]() {
-    issue(l_a, a_off, A_GROUPS, ca.kt, lds + (ca.issued % kStagesA) * STAGE_A);
+    issue(std::false_type{}, l_a, a_off, A_GROUPS, ca.kt, lds + (ca.issued % kStagesA) * STAGE_A);
     ++ca.issued;
   };
   auto issue_b = [&]() {
-    issue(l_b, b_off, B_GROUPS, cb.kt, lds + LDS_B0 + (cb.issued % kStagesB) * STAGE_B);
+    issue(std::integral_constant<bool, STREAM_B>{}, l_b, b_off, B_GROUPS, cb.kt,
+          lds + LDS_B0 + (cb.issued % kStagesB) * STAGE_B);
     ++cb.issued;
   };
   auto advance_a = [&]() {
     if (ca.issued >= total_steps) return;  // stay on the last step
-    if (++ca.kt == ca.kt_end) {
+    if (--ca.left == 0) {
       ca.item += walk.slots;
       setup_a(ca.item);
+    } else if (++ca.kt == ca.kt_end) {
+      ca.kt = ca.kt_begin;
     }
   };
   auto advance_b = [&]() {
     if (cb.issued >= total_steps) return;
-    if (++cb.kt == cb.kt_end) {
+    if (--cb.left == 0) {
       cb.item += walk.slots;
       setup_b(cb.item);
+    } else if (++cb.kt == cb.kt_end) {
+      cb.kt = cb.kt_begin;
     }
   };
 
@@ -717,7 +744,7 @@ void gemm_tiled_kernel(GemmParams p) {
         mfma_one(xa, xb, t, BLOCKSCALE || FIRST);
 #pragma unroll
         for (int l = 0; l < B_GROUPS; ++l)
-          if (l * NMFMA / B_GROUPS == t) load_chunk_to_lds(chunk_src(gb, b_off, l, real), wb + NW * l * 1024);
+          if (l * NMFMA / B_GROUPS == t) load_chunk_to_lds<STREAM_B>(chunk_src(gb, b_off, l, real), wb + NW * l * 1024);
 #pragma unroll
         for (int u = t * RPS; u < (t + 1) * RPS; ++u)
           if (u < NREAD) read_one(ya, yb, cur_a, cur_b, 1, u);
@@ -1288,26 +1315,38 @@ struct TileConfig {
   float us_per_step_alone;  // the same with at most one workgroup per CU
   float us_per_item;        // pipeline refill + epilogue of one work item
   float stream_bytes_per_us;  // operand bytes per microsecond the configuration can stream from HBM
+  float wg_stream_share;      // what one workgroup can stream, in units of 1/256 of that rate
 };
 constexpr int kNumTileConfigs = 4;
 constexpr int kNumGroupedTileConfigs = 3;  // the grouped form uses the first three
 // Measured on MI355X with normally distributed operands (clock under sustained MFMA load).
 constexpr TileConfig kTileConfigs[kNumTileConfigs] = {
-    {256, 256, tiled_wgs_per_cu(256, 256), 1.30f, 1.30f, 6.0f, 3.6e6f},
-    {128, 128, tiled_wgs_per_cu(128, 128), 1.00f, 0.62f, 5.0f, 4.4e6f},
-    {256, 128, tiled_wgs_per_cu(256, 128), 0.87f, 0.87f, 5.0f, 4.0e6f},
-    {64, 256, tiled_wgs_per_cu(64, 256), 0.75f, 0.75f, 7.0f, 4.8e6f},
+    {256, 256, tiled_wgs_per_cu(256, 256), 1.30f, 1.30f, 6.0f, 3.6e6f, 1.8f},
+    {128, 128, tiled_wgs_per_cu(128, 128), 1.00f, 0.60f, 5.0f, 4.4e6f, 1.18f},
+    {256, 128, tiled_wgs_per_cu(256, 128), 0.87f, 0.87f, 5.0f, 4.0e6f, 1.1f},
+    {64, 256, tiled_wgs_per_cu(64, 256), 0.75f, 0.75f, 9.0f, 5.0e6f, 2.0f},
 };
 
 // The skinny kernel's run time for comparison with the tiled plans at M <= 64: a fixed part
 // plus B streamed at a rate that falls with the number of 16-row blocks of A every workgroup
-// has to pull through L1 beside its rows of B (measured, MB per microsecond).
+// has to pull through L1 beside its rows of B (measured, MB per microsecond). With three or
+// four blocks the register budget leaves one workgroup per CU, and a last round of workgroups
+// that fills only part of the CUs streams at that fraction of the rate.
 inline float skinny_cost_us(int64_t M, int64_t N, int64_t K) {
-  static const float rate[4] = {7.0e6f, 4.5e6f, 4.2e6f, 3.9e6f};
+  static const float rate[4] = {6.0e6f, 4.5e6f, 3.44e6f, 3.6e6f};
   const int blocks = (int)((M + 15) / 16);
-  return 6.0f + (float)N * (float)K / rate[blocks < 1 ? 0 : blocks > 4 ? 3 : blocks - 1];
+  const int b = blocks < 1 ? 0 : blocks > 4 ? 3 : blocks - 1;
+  float r = rate[b];
+  if (b >= 2) {
+    const long wgs = (N + (b == 3 ? 31 : 15)) / (b == 3 ? 32 : 16);
+    const long rounds = (wgs + kNumCu - 1) / kNumCu;
+    r *= (float)wgs / (float)(rounds * kNumCu);
+  }
+  return 5.0f + (float)N * (float)K / r;
 }
 constexpr int kMaxSplits = 16;
+// Tile rows up to which a launch fetches B with the streaming policy (see gemm_tiled_kernel).
+constexpr int kStreamTileRows = 2;
 
 struct TiledPlan {
   int config, splits, steps_per_split;
@@ -1336,9 +1375,14 @@ inline float plan_cost_us(int64_t M, int64_t N, int64_t K, int config, int split
   const long full_rounds = items / slots, rest = items % slots;
   float t = full_rounds * (sps * c.us_per_step + c.us_per_item);
   if (rest) t += sps * (rest <= kNumCu ? c.us_per_step_alone : c.us_per_step) + c.us_per_item;
-  const float stream = ((float)M * (float)K + (float)N * (float)K) / c.stream_bytes_per_us;
+  // (one or two tile rows: B is fetched with the streaming policy, which is worth 8 %)
+  const bool streams_b = config != 0 && (M + c.bm - 1) / c.bm <= kStreamTileRows;
+  // (fewer work items than CUs: the busy CUs cannot make up for the idle ones beyond their share)
+  const float busy = items >= kNumCu ? 1.0f : fminf(1.0f, c.wg_stream_share * (float)items / (float)kNumCu);
+  const float stream =
+      ((float)M * (float)K + (float)N * (float)K) / (c.stream_bytes_per_us * (streams_b ? 1.08f : 1.0f) * busy);
   if (t < stream) t = stream;
-  if (splits > 1) t += 4.0f + 2.0f * (float)splits * (float)M * (float)N * 4.0f / 3.5e6f;
+  if (splits > 1) t += 3.0f + 2.0f * (float)splits * (float)M * (float)N * 4.0f / 5.0e6f;
   return t;
 }
 
@@ -1388,7 +1432,7 @@ int raise_lds_limit(const void* kernel, size_t lds_bytes, bool (&done)[kMaxDevic
 }
 
 template <int BM, int BN, int WAVES_M, int WAVES_N, bool KTAIL, int EPI, bool GROUPED = false, bool BLOCKSCALE = false,
-          int DIST = kDefaultDist>
+          int DIST = kDefaultDist, bool STREAM_B = false>
 int launch_tiled(GemmParams p, hipStream_t stream) {
   constexpr int threads = WAVES_M * WAVES_N * 64;
   constexpr size_t lds_bytes = tiled_lds_bytes(BM, BN, DIST);
@@ -1399,7 +1443,7 @@ int launch_tiled(GemmParams p, hipStream_t stream) {
   const long total = (long)p.tiles_m * p.tiles_n * p.splits;
   const long slots = (long)kNumCu * tiled_wgs_per_cu(BM, BN, BLOCKSCALE, DIST);
   long grid = total < slots ? ((total + kNumXcd - 1) / kNumXcd) * kNumXcd : slots;
-  auto kern = gemm_tiled_kernel<BM, BN, WAVES_M, WAVES_N, KTAIL, EPI, GROUPED, BLOCKSCALE, DIST>;
+  auto kern = gemm_tiled_kernel<BM, BN, WAVES_M, WAVES_N, KTAIL, EPI, GROUPED, BLOCKSCALE, DIST, STREAM_B>;
   static bool attr_done[kMaxDevices] = {};
   if (const int st = raise_lds_limit((const void*)kern, lds_bytes, attr_done)) return st;
   hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(threads), lds_bytes, stream, p);
@@ -1414,17 +1458,26 @@ int launch_tiled(GemmParams p, hipStream_t stream) {
   return MI355X_FP8_OK;
 }
 
-template <int BM, int BN, int WAVES_M, int WAVES_N, int DIST = kDefaultDist>
-int launch_tiled_config(const GemmParams& p, hipStream_t s) {
+template <int BM, int BN, int WAVES_M, int WAVES_N, bool STREAM_B>
+int launch_tiled_epilogue(const GemmParams& p, hipStream_t s) {
+  constexpr int D = kDefaultDist;
   const bool ktail = p.K % kStepK;
   if (p.splits > 1)
-    return ktail ? launch_tiled<BM, BN, WAVES_M, WAVES_N, true, kEpiPartial, false, false, DIST>(p, s)
-                 : launch_tiled<BM, BN, WAVES_M, WAVES_N, false, kEpiPartial, false, false, DIST>(p, s);
+    return ktail ? launch_tiled<BM, BN, WAVES_M, WAVES_N, true, kEpiPartial, false, false, D, STREAM_B>(p, s)
+                 : launch_tiled<BM, BN, WAVES_M, WAVES_N, false, kEpiPartial, false, false, D, STREAM_B>(p, s);
   if (p.bias)
-    return ktail ? launch_tiled<BM, BN, WAVES_M, WAVES_N, true, kEpiBias, false, false, DIST>(p, s)
-                 : launch_tiled<BM, BN, WAVES_M, WAVES_N, false, kEpiBias, false, false, DIST>(p, s);
-  return ktail ? launch_tiled<BM, BN, WAVES_M, WAVES_N, true, kEpiPlain, false, false, DIST>(p, s)
-               : launch_tiled<BM, BN, WAVES_M, WAVES_N, false, kEpiPlain, false, false, DIST>(p, s);
+    return ktail ? launch_tiled<BM, BN, WAVES_M, WAVES_N, true, kEpiBias, false, false, D, STREAM_B>(p, s)
+                 : launch_tiled<BM, BN, WAVES_M, WAVES_N, false, kEpiBias, false, false, D, STREAM_B>(p, s);
+  return ktail ? launch_tiled<BM, BN, WAVES_M, WAVES_N, true, kEpiPlain, false, false, D, STREAM_B>(p, s)
+               : launch_tiled<BM, BN, WAVES_M, WAVES_N, false, kEpiPlain, false, false, D, STREAM_B>(p, s);
+}
+
+template <int BM, int BN, int WAVES_M, int WAVES_N, bool MAY_STREAM>
+int launch_tiled_config(const GemmParams& p, hipStream_t s) {
+  if constexpr (MAY_STREAM) {
+    if ((p.M + BM - 1) / BM <= kStreamTileRows) return launch_tiled_epilogue<BM, BN, WAVES_M, WAVES_N, true>(p, s);
+  }
+  return launch_tiled_epilogue<BM, BN, WAVES_M, WAVES_N, false>(p, s);
 }
 
 template <int MT, int NTW, int DEPTH, int KW>
@@ -1545,10 +1598,11 @@ int mi355x_fp8_rowwise_gemm_ex(const void* a, const void* b, const float* a_scal
         p.steps_per_split = plan.steps_per_split;
         p.partial = plan.splits > 1 ? (float*)workspace : nullptr;
         switch (plan.config) {
-          case 0: return launch_tiled_config<256, 256, 2, 2>(p, s);
-          case 1: return launch_tiled_config<128, 128, 2, 2>(p, s);
-          case 2: return launch_tiled_config<256, 128, 2, 2>(p, s);
-          case 3: return launch_tiled_config<64, 256, 1, 4>(p, s);
+          // (256x256 tiles are never the plan for one or two tile rows)
+          case 0: return launch_tiled_config<256, 256, 2, 2, false>(p, s);
+          case 1: return launch_tiled_config<128, 128, 2, 2, true>(p, s);
+          case 2: return launch_tiled_config<256, 128, 2, 2, true>(p, s);
+          case 3: return launch_tiled_config<64, 256, 1, 4, true>(p, s);
           default: return fail(MI355X_FP8_EINVAL, "unknown tile configuration %d", plan.config);
         }
       }
