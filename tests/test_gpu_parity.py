@@ -317,7 +317,7 @@ def test_dispatch_is_pinned(gpu_device):
     assert ops.select_variant(48, 10240, 8192) == _lib.VARIANT_TILED
     assert ops.select_variant(64, 57344, 8192) == _lib.VARIANT_TILED
     assert ops.select_variant(32, 57344, 8192) == _lib.VARIANT_TILED
-    assert ops.select_variant(16, 57344, 8192) == _lib.VARIANT_SKINNY
+    assert ops.select_variant(16, 10240, 8192) == _lib.VARIANT_SKINNY
 
 
 def test_graph_capture_replays_match_eager(gpu_device):

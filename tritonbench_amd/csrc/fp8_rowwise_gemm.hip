@@ -1336,7 +1336,7 @@ inline float skinny_cost_us(int64_t M, int64_t N, int64_t K) {
   static const float rate[4] = {6.0e6f, 4.5e6f, 3.44e6f, 3.6e6f};
   const int blocks = (int)((M + 15) / 16);
   const int b = blocks < 1 ? 0 : blocks > 4 ? 3 : blocks - 1;
-  float r = rate[b];
+  float r = M <= 8 ? 7.2e6f : rate[b];  // (a few rows of A: its loads hit in L1 almost always)
   if (b >= 2) {
     const long wgs = (N + (b == 3 ? 31 : 15)) / (b == 3 ? 32 : 16);
     const long rounds = (wgs + kNumCu - 1) / kNumCu;
@@ -1379,8 +1379,9 @@ inline float plan_cost_us(int64_t M, int64_t N, int64_t K, int config, int split
   const bool streams_b = config != 0 && (M + c.bm - 1) / c.bm <= kStreamTileRows;
   // (fewer work items than CUs: the busy CUs cannot make up for the idle ones beyond their share)
   const float busy = items >= kNumCu ? 1.0f : fminf(1.0f, c.wg_stream_share * (float)items / (float)kNumCu);
-  const float stream =
-      ((float)M * (float)K + (float)N * (float)K) / (c.stream_bytes_per_us * (streams_b ? 1.08f : 1.0f) * busy);
+  // (64x256 tiles, at most two splits: the rotated K order lifts the rate further; priced cautiously)
+  const float policy = !streams_b ? 1.0f : (config == 3 && splits <= 2) ? 1.08f * 1.1f : 1.08f;
+  const float stream = ((float)M * (float)K + (float)N * (float)K) / (c.stream_bytes_per_us * policy * busy);
   if (t < stream) t = stream;
   if (splits > 1) t += 3.0f + 2.0f * (float)splits * (float)M * (float)N * 4.0f / 5.0e6f;
   return t;
