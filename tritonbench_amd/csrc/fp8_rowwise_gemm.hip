@@ -149,8 +149,9 @@ __device__ __forceinline__ void tile_coords(int t, int tiles_m, int tiles_n, int
 // tile's rows: 128 bytes per row = 8 chunks of 16 bytes, fetched from global memory as whole
 // 128-byte lines. Chunk c of row r sits at chunk position c ^ ((r >> 1) & 7): the MFMA
 // operand reads (consecutive lanes = consecutive rows, same logical chunk) then spread over
-// all banks. With the load distance of 2 steps that every instantiation uses A has two stages,
-// B three (2*32 KB + 3*32 KB = all 160 KB of a 256x256 tile's LDS). (A distance of 4 was
+// all banks. With a load distance of 2 steps A has two stages,
+// B three (2*32 KB + 3*32 KB = all 160 KB of a 256x256 tile's LDS); the 256x128 tile runs at a
+// distance of 3 (3*32 KB + 4*16 KB). (A distance of 4 was
 // measured on the 128x128 tile with one workgroup per CU and bought under 10 %: that tile is
 // bound by LDS bandwidth - its 64x64 wave tiles read 128 B/clk of operands - not by latency.)
 // ------------------------------------------------------------------------------------
@@ -1324,7 +1325,7 @@ constexpr TileConfig kTileConfigs[kNumTileConfigs] = {
     {256, 256, tiled_wgs_per_cu(256, 256), 1.30f, 1.30f, 6.0f, 3.6e6f, 1.8f},
     {128, 128, tiled_wgs_per_cu(128, 128), 1.00f, 0.60f, 5.0f, 4.4e6f, 1.18f},
     {256, 128, tiled_wgs_per_cu(256, 128), 0.87f, 0.87f, 5.0f, 4.0e6f, 1.1f},
-    {64, 256, tiled_wgs_per_cu(64, 256), 0.75f, 0.75f, 9.0f, 5.0e6f, 2.0f},
+    {64, 256, tiled_wgs_per_cu(64, 256), 0.75f, 0.75f, 9.0f, 5.7e6f, 1.42f},
 };
 
 // The skinny kernel's run time for comparison with the tiled plans at M <= 64: a fixed part
@@ -1461,7 +1462,10 @@ int launch_tiled(GemmParams p, hipStream_t stream) {
 
 template <int BM, int BN, int WAVES_M, int WAVES_N, bool STREAM_B>
 int launch_tiled_epilogue(const GemmParams& p, hipStream_t s) {
-  constexpr int D = kDefaultDist;
+  // 256x128 tiles have the LDS for loads three steps ahead (3 A + 4 B stages = 160 KB): worth 6-10 % where
+  // the operands come from HBM rather than the memory-side cache (M=1024, N=K=8192 cold: 65.9 -> 60.5 us;
+  // K=28672: 220 -> 199 us). The 64x256 tile measured 1-3 % slower that way and stays at two.
+  constexpr int D = (BM == 256 && BN == 128) ? 3 : kDefaultDist;
   const bool ktail = p.K % kStepK;
   if (p.splits > 1)
     return ktail ? launch_tiled<BM, BN, WAVES_M, WAVES_N, true, kEpiPartial, false, false, D, STREAM_B>(p, s)
@@ -1506,9 +1510,12 @@ const char* mi355x_fp8_rowwise_last_error(void) { return g_err; }
 int mi355x_fp8_rowwise_select_variant(int64_t M, int64_t N, int64_t K) {
   const int st = check_shape(M, N, K);
   if (st != MI355X_FP8_OK) return st;
-  // M <= 64: the streaming kernel, unless a tiled plan (64-row tiles, split K) is expected to
-  // beat it: long weight panels with three or four 16-row blocks of A
+  // M <= 64: the streaming kernel, unless a tiled plan (64- or 128-row tiles that stream B, split
+  // K where the tiles are few) is expected to beat it: from two 16-row blocks of A up on most
+  // shapes, with one block on the longest weight panels. Up to 8 rows the streaming kernel was
+  // never behind on any measured shape, so there the estimates are not consulted.
   if (M > kSkinnyMaxM) return MI355X_FP8_VARIANT_TILED;
+  if (M <= 8) return MI355X_FP8_VARIANT_SKINNY;
   return plan_tiled(M, N, K, -1, 0, kMaxSplits).cost_us < skinny_cost_us(M, N, K) ? MI355X_FP8_VARIANT_TILED
                                                                                  : MI355X_FP8_VARIANT_SKINNY;
 }
