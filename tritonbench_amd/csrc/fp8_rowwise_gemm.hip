@@ -1668,8 +1668,8 @@ int mi355x_fp8_rowwise_grouped_gemm(const void* a, const void* b, const float* a
     return ktail ? launch_tiled<256, 256, 2, 2, true, kEpiPlain, true>(p, s)
                  : launch_tiled<256, 256, 2, 2, false, kEpiPlain, true>(p, s);
   if (tile_config == 2)
-    return ktail ? launch_tiled<256, 128, 2, 2, true, kEpiPlain, true>(p, s)
-                 : launch_tiled<256, 128, 2, 2, false, kEpiPlain, true>(p, s);
+    return ktail ? launch_tiled<256, 128, 2, 2, true, kEpiPlain, true, false, 3>(p, s)
+                 : launch_tiled<256, 128, 2, 2, false, kEpiPlain, true, false, 3>(p, s);
   return ktail ? launch_tiled<128, 128, 2, 2, true, kEpiPlain, true>(p, s)
                : launch_tiled<128, 128, 2, 2, false, kEpiPlain, true>(p, s);
 }
