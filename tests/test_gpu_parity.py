@@ -97,6 +97,8 @@ PLAN_SHAPES = [
     # m, n, k, bias: ragged edges in both tile sizes, K tails, K shorter than the split count
     (130, 260, 128, True), (257, 129, 1040, False), (300, 520, 2048, True), (127, 1000, 4112, True),
     (512, 384, 640, False),
+    # many more tile columns than K steps: every start position of the rotated K order, tail step included
+    (100, 4000, 272, True),
 ]
 
 
