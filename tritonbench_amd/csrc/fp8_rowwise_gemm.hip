@@ -1339,6 +1339,8 @@ inline float skinny_cost_us(int64_t M, int64_t N, int64_t K) {
   const int blocks = (int)((M + 15) / 16);
   const int b = blocks < 1 ? 0 : blocks > 4 ? 3 : blocks - 1;
   float r = M <= 8 ? 7.2e6f : rate[b];  // (a few rows of A: its loads hit in L1 almost always)
+  // two blocks, one round of workgroups (two per CU) and a short K: everything is in flight at once
+  if (b == 1 && N <= 16 * 2 * kNumCu && K <= 8192) r = 4.9e6f;
   if (b >= 2) {
     const long wgs = (N + (b == 3 ? 31 : 15)) / (b == 3 ? 32 : 16);
     const long rounds = (wgs + kNumCu - 1) / kNumCu;
