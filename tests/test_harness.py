@@ -409,3 +409,42 @@ def test_export_dumps_inputs_and_outputs(tmp_path):
          "--export", "input", "--export-dir", str(tmp_path / "missing")])
     with pytest.raises(RuntimeError, match="must exist"):
         Op(tb_args=args, extra_args=extra).run(1, 1)
+
+
+def test_cuda_time_groups_kernels_between_flush_fills():
+    # per call: everything between two cache-clearing fills, whatever the number of kernels
+    # (upstream cuda_time.py:15-49 requires every kernel name to occur equally often instead)
+    from tritonbench_amd.harness.cuda_time import split_calls
+
+    fill = "void at::native::vectorized_elementwise_kernel<4, at::native::FillFunctor<int>, std::array<char*, 1ul> >(int)"
+    events = [
+        (5.0, 99.0, "stray kernel before the first fill"),
+        (10.0, 70.0, fill), (90.0, 20.0, "gemm"), (111.0, 6.0, "finalize"),
+        (120.0, 70.0, fill), (200.0, 22.0, "gemm"), (223.0, 5.0, "finalize"),
+        (230.0, 70.0, fill), (310.0, 14.0, "skinny"),
+    ]
+    assert split_calls(reversed(events)) == pytest.approx([0.026, 0.027, 0.014])
+    assert split_calls([]) == []
+
+
+def test_cuda_time_metric_needs_a_gpu_backend():
+    out = _run("--only", "ref", "--metrics", "cuda_time")
+    headers, table = out._table()
+    assert table[0][headers.index("ref-cuda_time")] == "not supported"
+
+
+@pytest.mark.gpu
+def test_cuda_time_metric_on_the_gpu(gpu_device):
+    from tritonbench_amd.harness.loader import load_opbench_by_name
+
+    Op = load_opbench_by_name("fp8_gemm_rowwise")
+    args, extra = get_parser().parse_known_args(
+        ["--op", "fp8_gemm_rowwise", "--m", "128", "--n", "8192", "--k", "8192", "--only", "_hip_mi355x",
+         "--metrics", "latency,cuda_time"])
+    op = Op(tb_args=args, extra_args=extra)
+    op.run(5, 20)
+    headers, table = op.output._table()
+    lat = table[0][headers.index("hip_mi355x-latency")]
+    dev = table[0][headers.index("hip_mi355x-cuda_time")]
+    # a split-K plan: two kernels per call, operands evicted before each, no launch gaps counted
+    assert 0.010 < dev.p50 < 0.100 and 0.010 < lat.p50 < 0.100

@@ -71,6 +71,7 @@ class BenchmarkOperatorMetrics:
     gpu_peak_mem: Optional[float] = None
     error_msg: Optional[str] = None
     hw_roofline: Optional[float] = None
+    cuda_time: Optional[Latency] = None
     extra_metrics: Optional[Dict[str, Any]] = None
 
 
@@ -389,6 +390,12 @@ class BenchmarkOperator(metaclass=_PostInit):
                 rec.tflops = self.tflops(fn_name, self.example_inputs, rec)
             if "hw_roofline" in want:
                 rec.hw_roofline = self.hw_roofline()
+            if "cuda_time" in want:
+                if backend_device == "cpu" or not torch.cuda.is_available():
+                    raise NotImplementedError("cuda_time needs a GPU backend")
+                from .cuda_time import do_bench_cuda_time
+
+                rec.cuda_time = do_bench_cuda_time(fn, warmup, rep)
             if "gpu_peak_mem" in want and self.device == "cuda":
                 torch.cuda.reset_peak_memory_stats()
                 fn()
