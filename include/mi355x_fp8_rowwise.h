@@ -126,6 +126,29 @@ int mi355x_fp8_rowwise_gemm_ex(const void* a, const void* b,
                                int variant, void* stream);
 
 /*
+ * mi355x_fp8_rowwise_gemm for callers that can neither allocate nor bring a workspace: code
+ * under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc. It has no
+ * counterpart in the reference (there every backend allocates through PyTorch). Same operands,
+ * same plan and bit-identical bf16 results as mi355x_fp8_rowwise_gemm called with a workspace of
+ * mi355x_fp8_rowwise_workspace_bytes(M, N, K, variant) bytes; the split-K partial sums go to a
+ * buffer of MI355X_FP8_NOALLOC_SCRATCH_BYTES built into the library's device code (one copy per
+ * GPU, held until the process ends). The call allocates and frees nothing.
+ *
+ * A plan that needs more than the buffer holds is refused with MI355X_FP8_ENOTSUP (use the
+ * workspace form for it); plans that need no workspace run at any size. All calls on one GPU
+ * share that GPU's buffer: calls that may overlap there (different streams, concurrently
+ * replayed graphs) race on it and must be ordered by the caller. The first call on a device
+ * looks the buffer's address up; make that call outside graph capture.
+ */
+#define MI355X_FP8_NOALLOC_SCRATCH_BYTES (64u << 20)
+int mi355x_fp8_rowwise_gemm_noalloc(const void* a, const void* b,
+                                    const float* a_scale, const float* b_scale,
+                                    const void* bias, void* c,
+                                    int64_t M, int64_t N, int64_t K,
+                                    int64_t lda, int64_t ldb, int64_t ldc,
+                                    int variant, void* stream);
+
+/*
  * Grouped form (mixture-of-experts layers): A and C are G row blocks stacked in one
  * matrix, block g holding m_sizes[g] rows; block g is multiplied with rows
  * [g*N, (g+1)*N) of B:

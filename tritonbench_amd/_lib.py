@@ -23,6 +23,7 @@ VARIANT_TILED = 1
 VARIANT_SKINNY = 2
 
 NUM_TILE_CONFIGS = 4
+NOALLOC_SCRATCH_BYTES = 64 << 20
 NUM_GROUPED_TILE_CONFIGS = 3
 
 
@@ -58,6 +59,11 @@ SIGNATURES = {
         [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int,
          c_int64, c_int64, c_int64, c_int64, c_int64, c_int64,
          c_void_p, c_size_t, c_int, c_void_p],
+    ),
+    "mi355x_fp8_rowwise_gemm_noalloc": (
+        c_int,
+        [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
+         c_int64, c_int64, c_int64, c_int64, c_int64, c_int64, c_int, c_void_p],
     ),
     "mi355x_fp8_rowwise_grouped_gemm": (
         c_int,

@@ -27,6 +27,7 @@
 #include <stdarg.h>
 #include <stdio.h>
 #include <string.h>
+#include <atomic>
 #include <type_traits>
 
 #include "../../include/mi355x_fp8_rowwise.h"
@@ -1502,6 +1503,33 @@ int launch_skinny(const GemmParams& p, hipStream_t stream) {
   return MI355X_FP8_OK;
 }
 
+// ---- built-in scratch of the entry point that allocates nothing
+// Split-K plans park their fp32 partial sums in device memory between the two launches. Callers
+// that cannot bring a workspace (HIP graph capture, serving loops that may not allocate) get this
+// array instead: every device the library is loaded on holds its own copy until the process
+// ends. In host code the array's name is only a handle for the symbol look-up below; kernels,
+// fills and copies take the per-device address that look-up returns.
+constexpr size_t kScratchBytes = (size_t)MI355X_FP8_NOALLOC_SCRATCH_BYTES;
+static __device__ __align__(256) unsigned char scratch[kScratchBytes];
+std::atomic<void*> g_scratch_ptr[kMaxDevices];
+
+// Address of the current device's copy of `scratch` (looked up once per device).
+int scratch_of_current_device(void** out) {
+  int dev = 0;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) return fail(MI355X_FP8_ELAUNCH, "hipGetDevice: %s", hipGetErrorString(e));
+  if (dev < 0 || dev >= kMaxDevices) return fail(MI355X_FP8_ENOTSUP, "device index %d beyond %d", dev, kMaxDevices - 1);
+  void* ptr = g_scratch_ptr[dev].load(std::memory_order_acquire);
+  if (!ptr) {
+    e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+    if (e != hipSuccess || !ptr)
+      return fail(MI355X_FP8_ELAUNCH, "hipGetSymbolAddress(scratch): %s", hipGetErrorString(e));
+    g_scratch_ptr[dev].store(ptr, std::memory_order_release);  // every thread finds the same address
+  }
+  *out = ptr;
+  return MI355X_FP8_OK;
+}
+
 }  // namespace
 
 extern "C" {
@@ -1628,6 +1656,30 @@ int mi355x_fp8_rowwise_gemm_ex(const void* a, const void* b, const float* a_scal
     default:
       return fail(MI355X_FP8_EINVAL, "unknown variant %d", variant);
   }
+}
+
+int mi355x_fp8_rowwise_gemm_noalloc(const void* a, const void* b, const float* a_scale, const float* b_scale,
+                                    const void* bias, void* c, int64_t M, int64_t N, int64_t K, int64_t lda,
+                                    int64_t ldb, int64_t ldc, int variant, void* stream) {
+  const int st = check_shape(M, N, K);
+  if (st != MI355X_FP8_OK) return st;
+  if (variant < 0 || (variant >> 24) || ((variant >> 8) & 0xff) > kNumTileConfigs)
+    return fail(MI355X_FP8_EINVAL, "unknown variant 0x%x", variant);
+  // host arithmetic only up to here: an oversized request is turned away before any device call
+  const size_t need = mi355x_fp8_rowwise_workspace_bytes(M, N, K, variant);
+  if (need > kScratchBytes)
+    return fail(MI355X_FP8_ENOTSUP,
+                "the plan for %lldx%lldx%lld needs %zu bytes of split-K scratch, the built-in buffer holds %zu; "
+                "call mi355x_fp8_rowwise_gemm with a workspace of that size instead",
+                (long long)M, (long long)N, (long long)K, need, kScratchBytes);
+  void* ws = nullptr;
+  if (need) {
+    if (const int ss = scratch_of_current_device(&ws)) return ss;
+  }
+  // Nothing in the buffer has to start at zero: every split stores its whole plane of partial sums
+  // before the finalize kernel (stream-ordered behind it) reads any of it.
+  return mi355x_fp8_rowwise_gemm_ex(a, b, a_scale, b_scale, bias, c, MI355X_FP8_OUT_BF16, M, N, K, lda, ldb, ldc,
+                                    ws, need ? kScratchBytes : 0, variant, stream);
 }
 
 int mi355x_fp8_rowwise_grouped_gemm(const void* a, const void* b, const float* a_scale, const float* b_scale,
