@@ -21,6 +21,7 @@ ELAUNCH = -3
 VARIANT_AUTO = 0
 VARIANT_TILED = 1
 VARIANT_SKINNY = 2
+SKINNY_ONE_TILE = 1 << 8  # skinny family: pins the one-tile-per-workgroup kernel
 
 NUM_TILE_CONFIGS = 4
 NOALLOC_SCRATCH_BYTES = 64 << 20

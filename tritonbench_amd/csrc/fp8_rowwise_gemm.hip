@@ -1095,6 +1095,188 @@ __global__ __launch_bounds__(KW * 64) void gemm_skinny_kernel(GemmParams p) {
 }
 
 // ------------------------------------------------------------------------------------
+// Persistent skinny kernel for M <= 16 and K = 16*SPW 128-byte steps (K = 2048 .. 8192): one
+// workgroup of 16 waves per CU walks a contiguous run of 16-row tiles of B. Wave w owns the K
+// steps w, w+16, ... of every tile and keeps its share of A (SPW fragments, 8 registers each)
+// in registers for the whole launch: A crosses the L2->L1 path once per CU instead of once per
+// tile, which is where the one-tile-per-workgroup kernel above loses a tenth of its time at
+// M = 16. The loads of B run one tile (SPW steps) ahead of their use; per tile the waves'
+// partial 16x16 results meet in LDS (two alternating areas, one barrier per tile) and one wave,
+// a different one for every tile, adds them in wave order and stores.
+// Workgroup g starts its K walk at step 2*(g/8) (workgroups g, g+8, ... share an XCD): the
+// workgroups of an XCD then ask its L2 for different lines of A at any one time, and the
+// addresses of B in flight do not all agree in their low bits (measured at N=K=8192, M=16:
+// 13.2 -> 12.7 us).
+// ------------------------------------------------------------------------------------
+constexpr int kPersistWaves = 16;
+
+// VEC: b_scale, bias and C are aligned for 16-, 8- and 8-byte accesses (else element by element).
+template <int SPW, bool VEC>
+__global__ __launch_bounds__(kPersistWaves * 64) void gemm_skinny_persistent_kernel(GemmParams p) {
+  constexpr int WAVES = kPersistWaves;
+  constexpr int STEPS = WAVES * SPW;
+  extern __shared__ __attribute__((aligned(1024))) uint8_t lds[];
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  uint8_t* buf = lds + wave * 2048;             // this wave's transpose buffer (one 16 x 128 B step)
+  v4f* red = (v4f*)(lds + WAVES * 2048);        // [2][WAVES][64] partial results
+
+  // this workgroup's run of tiles: the first `rem` workgroups take one tile more (quotient and
+  // remainder of tiles by workgroups come from the host: the division would sit in front of the
+  // first load)
+  const int g = blockIdx.x;
+  const int q = p.tiles_m, rem = p.tiles_n;
+  const int tile0 = g * q + min(g, rem);
+  const int count = q + (g < rem ? 1 : 0);
+  if (count <= 0) return;
+
+  // byte offset of this wave's i-th K step inside a row; wave-uniform, pinned to scalar registers
+  const int base_step = (wave + 2 * (g >> 3)) % STEPS;
+  uint32_t kofs[SPW];
+#pragma unroll
+  for (int i = 0; i < SPW; ++i) {
+    int s = base_step + WAVES * i;
+    if (s >= STEPS) s -= STEPS;
+    kofs[i] = (uint32_t)__builtin_amdgcn_readfirstlane(s * kStepK);
+  }
+  // a wave-uniform 64-bit offset pinned to scalar registers: loads then take the scalar-base +
+  // 32-bit lane-offset form instead of a 64-bit address pair per lane and load
+  auto uniform = [](size_t v) -> size_t {
+    const uint32_t lo = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)v);
+    const uint32_t hi = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)(v >> 32));
+    return ((size_t)hi << 32) | lo;
+  };
+  const int r16 = lane & 15, g4 = lane >> 4;
+  const int ld_row = lane >> 3, ld_c = lane & 7;
+  uint32_t b_lane[2];
+  int wr_off[2];
+#pragma unroll
+  for (int h = 0; h < 2; ++h) {
+    const int r = h * 8 + ld_row;
+    wr_off[h] = r * kStepK + ((ld_c ^ swz128(r)) * kChunk);
+    b_lane[h] = (uint32_t)r * (uint32_t)p.ldb + ld_c * kChunk;
+  }
+  const int rd0 = r16 * kStepK + (((2 * g4) ^ swz128(r16)) * kChunk);
+  const int rd1 = r16 * kStepK + (((2 * g4 + 1) ^ swz128(r16)) * kChunk);
+
+  v4i land[SPW][2];
+  const size_t tile_pitch = (size_t)16 * p.ldb;
+  size_t next_tile = uniform((size_t)tile0 * tile_pitch);  // byte offset of the tile the loads are at
+  auto fetch = [&](int i) {
+    const uint8_t* sbase = p.b + (next_tile + kofs[i]);
+#pragma unroll
+    for (int h = 0; h < 2; ++h) land[i][h] = __builtin_nontemporal_load((const v4i*)(sbase + b_lane[h]));
+  };
+  // The first tile's rows of B are asked for before anything else: they come from HBM.
+#pragma unroll
+  for (int i = 0; i < SPW; ++i) fetch(i);
+  __builtin_amdgcn_sched_barrier(0);
+  // A: whole-line loads (8 lanes per row, rows past M repeat the last one), turned into the
+  // MFMA lane layout through the transpose buffer, once
+  v8i fa[SPW];
+  {
+    v4i la[SPW][2];
+#pragma unroll
+    for (int i = 0; i < SPW; ++i) {
+      const uint8_t* sbase = p.a + kofs[i];
+#pragma unroll
+      for (int h = 0; h < 2; ++h)
+        la[i][h] = *(const v4i*)(sbase + ((uint32_t)min(h * 8 + ld_row, p.M - 1) * (uint32_t)p.lda + ld_c * kChunk));
+    }
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int i = 0; i < SPW; ++i) {
+      *(v4i*)(buf + wr_off[0]) = la[i][0];
+      *(v4i*)(buf + wr_off[1]) = la[i][1];
+      const v4i lo = *(const v4i*)(buf + rd0);
+      const v4i hi = *(const v4i*)(buf + rd1);
+      fa[i] = (v8i){lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+    }
+  }
+  // Wave w finishes the tiles j = w, w + 16, ... of the run: lane (m = lane % 16, quad lane / 16)
+  // owns C[m, 16*tile + 4*(lane/16) .. +3]. The column scales and bias of a wave's next tile are
+  // fetched long before they are used (here, and after each finished tile) and kept as loaded;
+  // a run without a tile for this wave reads the run's last tile instead.
+  const float fin_sa = p.a_scale[min(r16, p.M - 1)];
+  // Without a bias the same loads read the head of b_scale instead and the bits are masked off:
+  // the loads stay unconditional and in the global address space either way.
+  const uint16_t* const bias_src = p.bias ? p.bias : reinterpret_cast<const uint16_t*>(p.b_scale);
+  const int bias_stride = p.bias ? 1 : 0;
+  const uint16_t bias_mask = p.bias ? 0xffffu : 0u;
+  float sb_raw[4];
+  uint16_t bias_raw[4];
+  auto load_epi = [&](int j) {
+    const int n = (tile0 + min(j, count - 1)) * 16 + 4 * g4;
+    if (VEC) {
+      const v4f s4 = *(const v4f*)(p.b_scale + n);
+      const us4 b4 = *(const us4*)(bias_src + n * bias_stride);
+#pragma unroll
+      for (int x = 0; x < 4; ++x) sb_raw[x] = s4[x], bias_raw[x] = b4[x];
+    } else {
+#pragma unroll
+      for (int x = 0; x < 4; ++x) sb_raw[x] = p.b_scale[n + x], bias_raw[x] = bias_src[(n + x) * bias_stride];
+    }
+  };
+  load_epi(wave);
+
+  auto consume = [&](int i, v4f& acc) {
+    *(v4i*)(buf + wr_off[0]) = land[i][0];
+    *(v4i*)(buf + wr_off[1]) = land[i][1];
+    const v4i lo = *(const v4i*)(buf + rd0);
+    const v4i hi = *(const v4i*)(buf + rd1);
+    const v8i fb = (v8i){lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+    acc = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(fb, fa[i], acc, 0, 0, 0, 0, 0, 0);
+  };
+  auto finish = [&](int j, const v4f& acc) {
+    v4f* area = red + (j & 1) * WAVES * 64;
+    area[wave * 64 + lane] = acc;
+    __syncthreads();
+    // (the area is written again two tiles later, behind the next barrier, which the finishing
+    // wave reaches only after these reads)
+    if (wave == (j & (WAVES - 1))) {
+      v4f sum = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll 1
+      for (int w0 = 0; w0 < WAVES; w0 += 8) {  // eight partials in flight at a time: all sixteen cost 64 registers
+#pragma unroll
+        for (int w = 0; w < 8; ++w) sum += area[(w0 + w) * 64 + lane];
+      }
+      if (r16 < p.M) {
+        float r[4];
+#pragma unroll
+        for (int x = 0; x < 4; ++x) r[x] = __builtin_fmaf(sum[x] * fin_sa, sb_raw[x], bf16_to_f32(bias_raw[x] & bias_mask));
+        const uint32_t lo = pack_out_x2(r[0], r[1], p.out_f16), hi = pack_out_x2(r[2], r[3], p.out_f16);
+        uint16_t* dst = p.c + (size_t)r16 * p.ldc + (tile0 + j) * 16 + 4 * g4;
+        if (VEC) {
+          *(v2u*)dst = (v2u){lo, hi};
+        } else {
+          dst[0] = (uint16_t)lo; dst[1] = (uint16_t)(lo >> 16);
+          dst[2] = (uint16_t)hi; dst[3] = (uint16_t)(hi >> 16);
+        }
+      }
+      load_epi(j + WAVES);
+    }
+  };
+
+  int j = 0;
+  for (; j + 1 < count; ++j) {
+    next_tile = uniform(next_tile + tile_pitch);
+    v4f acc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int i = 0; i < SPW; ++i) {
+      consume(i, acc);
+      fetch(i);
+    }
+    finish(j, acc);
+  }
+  {
+    v4f acc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int i = 0; i < SPW; ++i) consume(i, acc);
+    finish(j, acc);
+  }
+}
+
+// ------------------------------------------------------------------------------------
 // Row-wise quantiser: one workgroup per row, two passes over the row (amax, then scale
 // and convert). e4m3fn encoding is done with integer arithmetic so the rounding
 // (nearest, ties to even, subnormals below 2^-6) does not depend on conversion hardware.
@@ -1335,7 +1517,10 @@ constexpr TileConfig kTileConfigs[kNumTileConfigs] = {
 // has to pull through L1 beside its rows of B (measured, MB per microsecond). With three or
 // four blocks the register budget leaves one workgroup per CU, and a last round of workgroups
 // that fills only part of the CUs streams at that fraction of the rate.
+inline bool persistent_skinny_fits(int64_t M, int64_t N, int64_t K);
 inline float skinny_cost_us(int64_t M, int64_t N, int64_t K) {
+  // the persistent form (measured: 12.7 us at N=K=8192, 71 us at N=57344)
+  if (persistent_skinny_fits(M, N, K)) return 3.0f + (float)N * (float)K / 6.9e6f;
   static const float rate[4] = {6.0e6f, 4.5e6f, 3.44e6f, 3.6e6f};
   const int blocks = (int)((M + 15) / 16);
   const int b = blocks < 1 ? 0 : blocks > 4 ? 3 : blocks - 1;
@@ -1530,6 +1715,38 @@ int scratch_of_current_device(void** out) {
   return MI355X_FP8_OK;
 }
 
+// The persistent skinny kernel takes M <= 16 with N a multiple of 16 and K of 2048 up to 8192.
+inline bool persistent_skinny_fits(int64_t M, int64_t N, int64_t K) {
+  return M <= 16 && N % 16 == 0 && K % (kPersistWaves * kStepK) == 0 && K / (kPersistWaves * kStepK) <= 4;
+}
+
+template <int SPW, bool VEC>
+int launch_skinny_persistent(const GemmParams& p, hipStream_t stream) {
+  constexpr size_t lds_bytes = (size_t)kPersistWaves * 2048 + 2 * kPersistWaves * 1024;
+  auto kern = gemm_skinny_persistent_kernel<SPW, VEC>;
+  static bool attr_done[kMaxDevices] = {};
+  if (const int st = raise_lds_limit((const void*)kern, lds_bytes, attr_done)) return st;
+  const long ntiles = p.N / 16;
+  const unsigned grid = (unsigned)(ntiles < kNumCu ? ntiles : kNumCu);
+  GemmParams q = p;
+  q.tiles_m = (int)(ntiles / grid);  // tiles per workgroup ...
+  q.tiles_n = (int)(ntiles % grid);  // ... and how many workgroups take one more
+  hipLaunchKernelGGL(kern, dim3(grid), dim3(kPersistWaves * 64), lds_bytes, stream, q);
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess) return fail(MI355X_FP8_ELAUNCH, "persistent skinny kernel launch: %s", hipGetErrorString(e));
+  return MI355X_FP8_OK;
+}
+
+template <bool VEC>
+int launch_skinny_persistent_steps(const GemmParams& p, hipStream_t s) {
+  switch (p.K / (kPersistWaves * kStepK)) {
+    case 1: return launch_skinny_persistent<1, VEC>(p, s);
+    case 2: return launch_skinny_persistent<2, VEC>(p, s);
+    case 3: return launch_skinny_persistent<3, VEC>(p, s);
+    default: return launch_skinny_persistent<4, VEC>(p, s);
+  }
+}
+
 }  // namespace
 
 extern "C" {
@@ -1649,6 +1866,12 @@ int mi355x_fp8_rowwise_gemm_ex(const void* a, const void* b, const float* a_scal
       // 16-row blocks of A | B tiles per wave | steps in flight per wave (sized to 128 VGPRs) | waves.
       // (Measured alternatives at M = 16: two B tiles per wave with 4, 6 or 8 steps in flight 17.8-19.9 us,
       // four waves 14.7-15.0 us, six steps in flight 16.4 us, against 14.4 us for this one.)
+      if (persistent_skinny_fits(M, N, K) && !(plan_bits & MI355X_FP8_SKINNY_ONE_TILE)) {
+        // 16-byte loads of b_scale, 8-byte loads of bias and 8-byte stores of C when everything is aligned for them
+        const bool vec = (reinterpret_cast<uintptr_t>(b_scale) & 15) == 0 && (reinterpret_cast<uintptr_t>(bias) & 7) == 0 &&
+                         (reinterpret_cast<uintptr_t>(c) & 7) == 0 && (ldc & 3) == 0;
+        return vec ? launch_skinny_persistent_steps<true>(p, s) : launch_skinny_persistent_steps<false>(p, s);
+      }
       if (M <= 16) return launch_skinny<1, 1, 4, 8>(p, s);
       if (M <= 32) return launch_skinny<2, 1, 2, 8>(p, s);
       if (M <= 48) return launch_skinny<3, 1, 2, 8>(p, s);
