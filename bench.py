@@ -1,21 +1,26 @@
 """Benchmark of the row-wise FP8 GEMM hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--all-configs] [--no-cpu-baseline]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu-baseline] [--no-extra]
 
-The defaults (100 warm-up, 400 timed steps, about 0.2 s of GPU time) are long enough for the
-GPU's clock governor to settle: the first few milliseconds of a burst run well below the
-sustained clock, so a handful of steps under-reports throughput by 20-30 %.
+One step = one pass of the hot path (one mi355x_fp8_rowwise_gemm call through the C ABI) over
+the headline workload M=N=K=8192 with operands resident in HBM. Prints ONE JSON line: the
+headline TFLOP/s, the roofline of the dominant kernel measured with HIP events on the launch
+stream, the CPU baseline (the oracle's fp32 dequantise + torch.matmul, timed on this machine's
+host cores), the HBM-bound headline (M=16) with a roofline block of its own, and under
+"configs" one row per benchmark configuration (microseconds, TFLOP/s, GB/s, bound, fraction of
+that bound's peak): the decode shape, all twenty Llama-3-70B projection shapes, the two ragged
+shapes with bias (each of these with its own CPU baseline where that takes seconds), and the
+neighbouring kernels (grouped, block-scaled, quantiser).
 
-One step = one pass of the hot path (one mi355x_fp8_rowwise_gemm call through the C ABI)
-over the headline workload M=N=K=8192 with operands resident in HBM. Prints ONE JSON line:
-the headline TFLOP/s, the roofline of the dominant kernel measured with HIP events on the
-launch stream, the CPU baseline (the oracle's fp32 dequantise + torch.matmul, timed on this
-machine's host cores), and per-configuration figures for the skinny (HBM-bound) and the
-other benchmark shapes under "configs".
+The device runs its first milliseconds of matrix work after an idle spell well below the
+sustained clock, so whatever --warmup says the workload is launched untimed for --preheat-ms
+first; the K timed steps follow at once.
 """
 import argparse
+import hashlib
 import json
 import os
+import statistics
 import sys
 import time
 
@@ -27,118 +32,167 @@ sys.path.insert(0, ROOT)
 PEAK_FP8_TFLOPS = 5000.0  # dense FP8 MFMA, MI355X datasheet
 PEAK_HBM_GBPS = 8000.0    # HBM3E, MI355X datasheet
 SEED = 1337
-TILED_8192_TRAFFIC_BYTES = (790326 + 131841) * 1024
+KERNEL_SOURCE = os.path.join(ROOT, "tritonbench_amd", "csrc", "fp8_rowwise_gemm.hip")
+TRAFFIC_FILES = {  # written by `python -m tritonbench_amd.harness.traffic` from two rocprofv3 counter passes
+    "tiled": os.path.join(ROOT, "profiles", "tiled_8192cubed_traffic.json"),
+    "skinny": os.path.join(ROOT, "profiles", "skinny_16x8192x8192_traffic.json"),
+}
+LLAMA3_70B_NK = [(10240, 8192), (8192, 8192), (57344, 8192), (8192, 28672)]
+LLAMA3_70B_M = [1, 32, 128, 1024, 4096]
 
 
-def make_device_inputs(m, n, k, sigma, bias, dev, copies=1):
-    """Seeded synthetic operands generated and quantised on the device (the HIP quantiser is
-    bit-exact against the oracle). `copies` > 1 returns independent operand sets to rotate
-    through so that no call finds its operands in L2 or the 256 MB memory-side cache."""
+def source_sha() -> str:
+    with open(KERNEL_SOURCE, "rb") as f:
+        return hashlib.sha256(f.read()).hexdigest()[:16]
+
+
+def measured_traffic(which: str):
+    """HBM-side bytes per launch from the committed counter summary, or None. The summary names
+    the kernel source it was measured on: a figure from an older source is still reported, marked
+    stale, so that it cannot pass for a measurement of the present kernel."""
+    path = TRAFFIC_FILES[which]
+    if not os.path.exists(path):
+        return None, {"traffic_source": None}
+    with open(path) as f:
+        t = json.load(f)
+    note = {"traffic_source": os.path.relpath(path, ROOT), "traffic_kernel": t.get("kernel"),
+            "traffic_stale": t.get("source_sha") != source_sha()}
+    return t.get("traffic_bytes"), note
+
+
+def _generator(dev, *key):
+    g = torch.Generator(device=dev)
+    g.manual_seed(SEED + sum(int(k) * w for k, w in zip(key, (7, 3, 1, 11))))
+    return g
+
+
+def make_weights(n, k, sigma, bias, dev, copies):
+    """`copies` independent (wq, w_scale, bias) sets, generated and quantised on the device (the
+    HIP quantiser is bit-exact against the oracle)."""
     from tritonbench_amd import ops
 
-    g = torch.Generator(device=dev)
-    g.manual_seed(SEED + m * 7 + n * 3 + k)
+    g = _generator(dev, 0, n, k)
     sets = []
     for _ in range(copies):
-        x = torch.randn((m, k), generator=g, device=dev, dtype=torch.float32) * sigma
         w = torch.randn((n, k), generator=g, device=dev, dtype=torch.float32) * sigma
-        xq, xs = ops.fp8_row_quantize(x)
         wq, ws = ops.fp8_row_quantize(w)
-        del x, w
+        del w
         b = (0.1 * torch.randn((n,), generator=g, device=dev, dtype=torch.float32)).to(torch.bfloat16) if bias else None
-        out = torch.empty((m, n), dtype=torch.bfloat16, device=dev)
-        sets.append((xq, wq, xs, ws, b, out))
-    global _workspace
-    _workspace = ops.gemm_workspace(m, n, k, dev)  # split-K partial sums, when the plan has them
+        sets.append((wq, ws, b))
     return sets
 
 
-_workspace = None
-
-
-def preheat(sets, ms):
-    """Untimed launches of the workload for about `ms` milliseconds. After idling the device runs
-    its first 15-20 ms of matrix work at a lower clock (8192^3: 474 us per launch against 405 us in
-    the steady state on the same device); a short --warmup would leave part of that ramp inside
-    the timed region."""
-    import time
+def make_sets(m, weights, sigma, dev):
+    """One operand set per weight copy: (xq, wq, x_scale, w_scale, bias, out). Rotating through
+    sets larger than the caches means no call finds its operands in L2 or the 256 MB memory-side
+    cache."""
     from tritonbench_amd import ops
 
-    t0 = time.perf_counter()
+    n, k = weights[0][0].shape
+    g = _generator(dev, m, n, k)
+    sets = []
+    for (wq, ws, b) in weights:
+        x = torch.randn((m, k), generator=g, device=dev, dtype=torch.float32) * sigma
+        xq, xs = ops.fp8_row_quantize(x)
+        sets.append((xq, wq, xs, ws, b, torch.empty((m, n), dtype=torch.bfloat16, device=dev)))
+    return sets, ops.gemm_workspace(m, n, k, dev)
+
+
+def copies_for(n, k, cap=8):
+    """Operand sets needed for the rotation to out-run the 256 MB memory-side cache."""
+    return max(2, min(cap, int(600e6 // (n * k)) + 1))
+
+
+def launch(s, workspace):
+    from tritonbench_amd import ops
+
+    xq, wq, xs, ws, b, out = s
+    ops.fp8_gemm_rowwise(xq, wq, xs, ws, bias=b, out=out, workspace=workspace)
+
+
+def preheat(sets, workspace, ms):
+    """Untimed launches of the workload for about `ms` milliseconds of wall time."""
+    t0, i = time.perf_counter(), 0
     while (time.perf_counter() - t0) * 1e3 < ms:
-        for i in range(10):
-            xq, wq, xs, ws, b, out = sets[i % len(sets)]
-            ops.fp8_gemm_rowwise(xq, wq, xs, ws, bias=b, out=out, workspace=_workspace)
+        for _ in range(10):
+            launch(sets[i % len(sets)], workspace)
+            i += 1
         torch.cuda.synchronize()
 
 
-def time_steps(sets, steps, warmup):
+def time_steps(sets, workspace, steps, warmup):
     """Average ms per call over exactly `steps` calls, HIP events on the launch stream."""
-    from tritonbench_amd import ops
-
     stream = torch.cuda.current_stream()
     for i in range(warmup):
-        xq, wq, xs, ws, b, out = sets[i % len(sets)]
-        ops.fp8_gemm_rowwise(xq, wq, xs, ws, bias=b, out=out, workspace=_workspace)
-    torch.cuda.synchronize()
+        launch(sets[i % len(sets)], workspace)
     start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
     start.record(stream)
     for i in range(steps):
-        xq, wq, xs, ws, b, out = sets[i % len(sets)]
-        ops.fp8_gemm_rowwise(xq, wq, xs, ws, bias=b, out=out, workspace=_workspace)
+        launch(sets[i % len(sets)], workspace)
     end.record(stream)
     torch.cuda.synchronize()
     return start.elapsed_time(end) / steps
 
 
-def time_steps_graph(sets, steps, warmup, min_replay_ms=6.0, preheat_ms=30.0):
-    """Same, with the calls captured in one HIP graph (no per-launch host gaps); this is how the
-    benchmark harness times the operator. The graph holds at least `steps` calls and enough of
-    them for a replay to last `min_replay_ms`; replays run untimed for `preheat_ms` first (the
-    device clock needs that after an idle spell), then the best of three timed replays counts."""
-    import time
-    from tritonbench_amd import ops
-
+def time_graph(call, steps, min_replay_ms=6.0, preheat_ms=30.0, replays=5):
+    """ms per call of call(i) with the calls captured in one HIP graph (no per-launch host gaps:
+    how the benchmark harness times the operator). The graph holds at least `steps` calls and
+    enough of them for a replay to last `min_replay_ms`; replays run untimed for `preheat_ms`
+    first. Returns (best, median) over `replays` timed replays."""
     side = torch.cuda.Stream()
     with torch.cuda.stream(side):
-        for i in range(max(warmup, 1)):
-            xq, wq, xs, ws, b, out = sets[i % len(sets)]
-            ops.fp8_gemm_rowwise(xq, wq, xs, ws, bias=b, out=out, workspace=_workspace)
+        call(0)
         torch.cuda.synchronize()
         t0 = time.perf_counter()
         for i in range(5):
-            xq, wq, xs, ws, b, out = sets[i % len(sets)]
-            ops.fp8_gemm_rowwise(xq, wq, xs, ws, bias=b, out=out, workspace=_workspace)
+            call(i)
         torch.cuda.synchronize()
         est_ms = max((time.perf_counter() - t0) * 1e3 / 5, 1e-3)
         steps = int(min(max(steps, min_replay_ms / est_ms), 2000))
         g = torch.cuda.CUDAGraph()
         with torch.cuda.graph(g, stream=side):
             for i in range(steps):
-                xq, wq, xs, ws, b, out = sets[i % len(sets)]
-                ops.fp8_gemm_rowwise(xq, wq, xs, ws, bias=b, out=out, workspace=_workspace)
+                call(i)
         torch.cuda.synchronize()
         t0 = time.perf_counter()
         while (time.perf_counter() - t0) * 1e3 < preheat_ms:
             g.replay()
             torch.cuda.synchronize()
-        best = None
-        for _ in range(3):
+        times = []
+        for _ in range(replays):
             start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
             start.record(side)
             g.replay()
             end.record(side)
             torch.cuda.synchronize()
-            ms = start.elapsed_time(end) / steps
-            best = ms if best is None else min(best, ms)
-    return best
+            times.append(start.elapsed_time(end) / steps)
+    return min(times), statistics.median(times)
+
+
+def figures(m, n, k, bias, ms, ms_median=None):
+    flops = 2 * m * n * k + (2 * m * n if bias else 0)
+    nbytes = m * k + n * k + 2 * m * n
+    tflops = flops / ms / 1e9
+    gbps = nbytes / ms / 1e6
+    t_mfma = flops / (PEAK_FP8_TFLOPS * 1e12)
+    t_hbm = nbytes / (PEAK_HBM_GBPS * 1e9)
+    bound = "mfma" if t_mfma >= t_hbm else "hbm"
+    frac = tflops / PEAK_FP8_TFLOPS if bound == "mfma" else gbps / PEAK_HBM_GBPS
+    row = dict(us=ms * 1e3, tflops=tflops, gbps=gbps, bound=bound, frac=frac)
+    if ms_median is not None:
+        row["us_median"] = ms_median * 1e3
+    return row
+
+
+def gemm_row(m, sets, workspace, steps):
+    xq, wq, _, _, b, _ = sets[0]
+    best, med = time_graph(lambda i: launch(sets[i % len(sets)], workspace), steps)
+    return figures(m, wq.shape[0], wq.shape[1], b is not None, best, med)
 
 
 def timed_calls(call, steps, preheat_ms=30.0):
     """ms per call of call(i) over `steps` calls (HIP events on the launch stream), after untimed
-    calls for `preheat_ms` so the device clock has settled."""
-    import time
-
+    calls for `preheat_ms`."""
     t0, i = time.perf_counter(), 0
     while (time.perf_counter() - t0) * 1e3 < preheat_ms:
         for _ in range(5):
@@ -160,8 +214,7 @@ def time_quantiser(r, k, dtype, dev, steps=60, copies=3):
     output + one f32 scale per row; sources rotate so no call finds its row in a cache."""
     from tritonbench_amd import ops
 
-    g = torch.Generator(device=dev)
-    g.manual_seed(SEED + r + k)
+    g = _generator(dev, r, k)
     xs = [torch.randn((r, k), generator=g, device=dev, dtype=torch.float32).to(dtype) for _ in range(copies)]
     ms = timed_calls(lambda i: ops.fp8_row_quantize(xs[i % copies]), steps)
     nbytes = r * k * (xs[0].element_size() + 1) + 4 * r
@@ -173,14 +226,14 @@ def time_grouped(g, m, n, k, dev, steps=40, copies=2):
     flops = 2*M*N*K, bytes = M*K + G*N*K + 2*M*N."""
     from tritonbench_amd import ops
 
-    gen = torch.Generator(device=dev)
-    gen.manual_seed(SEED + g + m + n + k)
+    gen = _generator(dev, g, m, n, k)
     sets = []
     for _ in range(copies):
         xq, xs = ops.fp8_row_quantize(torch.randn((m, k), generator=gen, device=dev, dtype=torch.float32))
         wq, ws = ops.fp8_row_quantize(torch.randn((g * n, k), generator=gen, device=dev, dtype=torch.float32))
         sets.append((xq, wq, xs, ws, torch.zeros((m, n), dtype=torch.bfloat16, device=dev)))
     sizes = torch.tensor([m // g] * g, dtype=torch.int32, device=dev)
+
     def call(i):
         xq, wq, xs, ws, out = sets[i % copies]
         ops.fp8_gemm_rowwise_grouped(xq, wq, sizes, xs, ws, out=out)
@@ -197,8 +250,7 @@ def time_blockwise(m, n, k, dev, steps=30):
     from tritonbench_amd import ops
     from tritonbench_amd.operators.fp8_gemm_blockwise.operator import fp8_block_quantize
 
-    gen = torch.Generator(device=dev)
-    gen.manual_seed(SEED + 5 * m + n + k)
+    gen = _generator(dev, 5 * m, n, k)
     xq, xs = fp8_block_quantize(torch.randn((m, k), generator=gen, device=dev, dtype=torch.float32))
     wq, ws = fp8_block_quantize(torch.randn((n, k), generator=gen, device=dev, dtype=torch.float32))
     out = torch.empty((m, n), dtype=torch.bfloat16, device=dev)
@@ -208,45 +260,68 @@ def time_blockwise(m, n, k, dev, steps=30):
                 frac=flops / ms / 1e9 / PEAK_FP8_TFLOPS)
 
 
-def figures(m, n, k, bias, ms):
-    flops = 2 * m * n * k + (2 * m * n if bias else 0)
-    nbytes = m * k + n * k + 2 * m * n
-    tflops = flops / ms / 1e9
-    gbps = nbytes / ms / 1e6
-    t_mfma = flops / (PEAK_FP8_TFLOPS * 1e12)
-    t_hbm = nbytes / (PEAK_HBM_GBPS * 1e9)
-    bound = "mfma" if t_mfma >= t_hbm else "hbm"
-    frac = tflops / PEAK_FP8_TFLOPS if bound == "mfma" else gbps / PEAK_HBM_GBPS
-    return dict(us=ms * 1e3, tflops=tflops, gbps=gbps, bound=bound, frac=frac)
-
-
-def cpu_baseline(xq, wq, xs, ws, budget_s=12.0):
+def cpu_baseline(s, what, budget_s=12.0, max_calls=5):
     """The oracle (fp32 dequantise + torch.matmul) on host cores, on the same operands."""
     from oracle import fp8_rowwise as orc
 
+    xq, wq, xs, ws, b, _ = s
     hxq, hwq, hxs, hws = xq.cpu(), wq.cpu(), xs.cpu(), ws.cpu()
+    hb = None if b is None else b.cpu()
     m, k = hxq.shape
     n = hwq.shape[0]
     t0 = time.perf_counter()
-    orc.dequant_matmul(hxq, hwq, hxs, hws)  # warm-up (also pages in the BLAS)
+    orc.dequant_matmul(hxq, hwq, hxs, hws, hb)  # warm-up (also pages in the BLAS)
     first = time.perf_counter() - t0
-    times = []
-    spent = 0.0
-    while spent < budget_s and len(times) < 5:
+    times, spent = [], 0.0
+    while spent < budget_s and len(times) < max_calls:
         t0 = time.perf_counter()
-        orc.dequant_matmul(hxq, hwq, hxs, hws)
+        orc.dequant_matmul(hxq, hwq, hxs, hws, hb)
         dt = time.perf_counter() - t0
         times.append(dt)
         spent += dt
     best = min(times) if times else first
+    flops = 2 * m * n * k + (2 * m * n if b is not None else 0)
     return {
-        "value": 2 * m * n * k / best / 1e12,
+        "value": flops / best / 1e12,
         "unit": "TFLOP/s",
+        "gbps": (m * k + n * k + 2 * m * n) / best / 1e9,
+        "ms": best * 1e3,
         "cores": torch.get_num_threads(),
         "kind": "port",
-        "sample": f"full M=N=K=8192 workload, best of {len(times)} calls after 1 warm-up ({best:.3f} s/call, "
+        "sample": f"full {what} workload, best of {len(times)} calls after 1 warm-up ({best:.4f} s/call, "
                   f"dequantise included, host cpu_count {os.cpu_count()})",
     }
+
+
+def profile_kernel(which, dev):
+    """A short run of one kernel's workload for rocprofv3 counter passes, preceded by a copy
+    kernel of known size (an elementwise multiply of a 256 MiB tensor: reads it once, writes as
+    much) that the counter readings are scaled by."""
+    cal = torch.ones((8192, 8192), dtype=torch.float32, device=dev)
+    for _ in range(3):
+        cal.mul(2.0)
+    torch.cuda.synchronize()
+    if which == "tiled":
+        sets, wsp = make_sets(8192, make_weights(8192, 8192, 1.0, False, dev, 1), 1.0, dev)
+        fig = figures(8192, 8192, 8192, False, time_steps(sets, wsp, 20, 5))
+    elif which == "skinny":
+        sets, wsp = make_sets(16, make_weights(8192, 8192, 1.0, False, dev, 10), 1.0, dev)
+        fig = figures(16, 8192, 8192, False, time_steps(sets, wsp, 40, 10))
+    elif which == "quantise":
+        fig = {"f32": time_quantiser(8192, 8192, torch.float32, dev, steps=20),
+               "bf16": time_quantiser(8192, 8192, torch.bfloat16, dev, steps=20)}
+    elif which == "grouped":
+        fig = time_grouped(4, 8192, 4096, 4096, dev, steps=20)
+    elif which == "decode128":
+        sets, wsp = make_sets(128, make_weights(8192, 8192, 0.02, False, dev, 8), 0.02, dev)
+        fig = figures(128, 8192, 8192, False, time_steps(sets, wsp, 40, 10))
+    elif which == "ragged":
+        sets, wsp = make_sets(1000, make_weights(3000, 4112, 1.0, True, dev, 2), 1.0, dev)
+        fig = figures(1000, 3000, 4112, True, time_steps(sets, wsp, 40, 10))
+    else:
+        raise ValueError(which)
+    print(json.dumps({"profile_kernel": which, "figures": fig, "source_sha": source_sha(),
+                      "calibration": {"kernel": "MulFunctor", "read_bytes": cal.numel() * 4, "write_bytes": cal.numel() * 4}}))
 
 
 def main():
@@ -254,12 +329,11 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=400)
     ap.add_argument("--warmup", type=int, default=100)
-    ap.add_argument("--preheat-ms", type=float, default=80.0,
+    ap.add_argument("--preheat-ms", type=float, default=300.0,
                     help="untimed launches before the warmup steps, until the device clock has settled")
-    ap.add_argument("--all-configs", action="store_true", help="also time every Llama-3-70B projection shape")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-extra", action="store_true", help="headline workload only")
-    ap.add_argument("--profile-kernel", choices=["skinny", "quantise", "grouped"],
+    ap.add_argument("--profile-kernel", choices=["tiled", "skinny", "quantise", "grouped", "decode128", "ragged"],
                     help="run only that kernel's workload a few times (for rocprofv3 counter passes) and print its figures")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
@@ -276,23 +350,16 @@ def main():
     torch.cuda.set_device(dev)
 
     if args.profile_kernel:
-        if args.profile_kernel == "skinny":
-            ps = make_device_inputs(16, 8192, 8192, 1.0, False, dev, copies=10)
-            fig = figures(16, 8192, 8192, False, time_steps(ps, 40, 10))
-        elif args.profile_kernel == "quantise":
-            fig = {"f32": time_quantiser(8192, 8192, torch.float32, dev, steps=20),
-                   "bf16": time_quantiser(8192, 8192, torch.bfloat16, dev, steps=20)}
-        else:
-            fig = time_grouped(4, 8192, 4096, 4096, dev, steps=20)
-        print(json.dumps({"profile_kernel": args.profile_kernel, "figures": fig}))
+        profile_kernel(args.profile_kernel, dev)
         return
 
     m = n = k = 8192
-    sets = make_device_inputs(m, n, k, 1.0, False, dev, copies=1)
+    head_sets, head_ws = make_sets(m, make_weights(n, k, 1.0, False, dev, 1), 1.0, dev)
     torch.cuda.synchronize()
-    preheat(sets, args.preheat_ms)
-    ms = time_steps(sets, args.steps, args.warmup)
+    preheat(head_sets, head_ws, args.preheat_ms)
+    ms = time_steps(head_sets, head_ws, args.steps, args.warmup)
     head = figures(m, n, k, False, ms)
+    traffic, traffic_note = measured_traffic("tiled")
 
     line = {
         "metric": "fp8_gemm_rowwise TFLOP/s at M=N=K=8192 (1 GPU)",
@@ -315,51 +382,65 @@ def main():
             "peak": PEAK_FP8_TFLOPS,
             "unit": "TFLOP/s",
             "frac": head["tflops"] / PEAK_FP8_TFLOPS,
-            # HBM-side bytes per launch of the dominant kernel, from rocprofv3 --pmc FETCH_SIZE /
-            # WRITE_SIZE scaled by a copy kernel of known size (FETCH x2.0, WRITE x1.0); a property
-            # of the kernel's tile walk on this workload, re-profiled whenever the kernel changes
-            "traffic": TILED_8192_TRAFFIC_BYTES,
+            # HBM-side bytes per launch of the dominant kernel from two rocprofv3 counter passes
+            # (FETCH_SIZE, WRITE_SIZE), each scaled by a copy kernel of known size in the same run
+            "traffic": traffic,
+            **traffic_note,
         },
     }
 
     if not args.no_extra:
         configs = {}
+        cpu = not args.no_cpu_baseline
         # C3: decode-sized, HBM-bound. Cold = rotate through operand sets larger than every cache.
         cm, cn, ck = 16, 8192, 8192
-        cold_sets = make_device_inputs(cm, cn, ck, 1.0, False, dev, copies=10)
-        cold = figures(cm, cn, ck, False, time_steps_graph(cold_sets, 200, 5))
-        warm = figures(cm, cn, ck, False, time_steps_graph(cold_sets[:1], 200, 5))
+        cold_sets, cws = make_sets(cm, make_weights(cn, ck, 1.0, False, dev, 10), 1.0, dev)
+        cold = gemm_row(cm, cold_sets, cws, 200)
+        warm = gemm_row(cm, cold_sets[:1], cws, 200)
         configs["c3_skinny_16x8192x8192"] = {"cold": cold, "cache_resident": warm}
+        if cpu:
+            configs["c3_skinny_16x8192x8192"]["cpu_baseline"] = cpu_baseline(cold_sets[0], "M=16, N=K=8192", budget_s=4.0)
         del cold_sets
+        straffic, snote = measured_traffic("skinny")
         line["hbm_metric"] = {
             "metric": "fp8_gemm_rowwise HBM GB/s at M=16,N=K=8192 (cold operands)",
-            "value": cold["gbps"], "unit": "GB/s", "frac": cold["gbps"] / PEAK_HBM_GBPS,
+            "value": cold["gbps"], "unit": "GB/s", "us": cold["us"], "us_median": cold["us_median"],
+            "roofline": {"bound": "hbm", "achieved": cold["gbps"], "peak": PEAK_HBM_GBPS, "unit": "GB/s",
+                         "frac": cold["gbps"] / PEAK_HBM_GBPS, "traffic": straffic, **snote},
         }
+        # C5: ragged shapes with fused bias
         for (rm, rn, rk) in [(1000, 3000, 4112), (4097, 7168, 2048)]:
-            rs = make_device_inputs(rm, rn, rk, 1.0, True, dev, copies=2)
-            configs[f"c5_ragged_bias_{rm}x{rn}x{rk}"] = figures(rm, rn, rk, True, time_steps_graph(rs, 50, 3))
+            rs, rws = make_sets(rm, make_weights(rn, rk, 1.0, True, dev, 2), 1.0, dev)
+            name = f"c5_ragged_bias_{rm}x{rn}x{rk}"
+            configs[name] = gemm_row(rm, rs, rws, 50)
+            if cpu:
+                configs[name]["cpu_baseline"] = cpu_baseline(rs[0], f"{rm}x{rn}x{rk} + bias", budget_s=4.0, max_calls=3)
             del rs
-        make_device_inputs(m, n, k, 1.0, False, dev, copies=0)  # workspace of the headline plan again
-        configs["c2_square_8192_graph"] = figures(m, n, k, False, time_steps_graph(sets, 20, 2))
+        configs["c2_square_8192_graph"] = gemm_row(m, head_sets, head_ws, 20)
+        # C1: the reference's CPU-runnable plumbing case, here on the device with the host figure beside it
+        ps, pws = make_sets(128, make_weights(256, 512, 1.0, False, dev, 1), 1.0, dev)
+        configs["c1_plumbing_128x256x512"] = gemm_row(128, ps, pws, 200)
+        if cpu:
+            configs["c1_plumbing_128x256x512"]["cpu_baseline"] = cpu_baseline(ps[0], "128x256x512", budget_s=1.0)
+        # C4: Llama-3-70B projections, sigma 0.02; the weight copies of an (N, K) pair serve its whole M sweep
+        for (ln, lk) in LLAMA3_70B_NK:
+            weights = make_weights(ln, lk, 0.02, False, dev, copies_for(ln, lk))
+            for lm in LLAMA3_70B_M:
+                ls, lws = make_sets(lm, weights, 0.02, dev)
+                configs[f"c4_llama70b_{lm}x{ln}x{lk}"] = gemm_row(lm, ls, lws, 30 if lm < 1024 else 10)
+                del ls, lws
+            del weights
+            torch.cuda.empty_cache()
         configs["grouped_g4_8192x4096x4096"] = time_grouped(4, 8192, 4096, 4096, dev)
         configs["grouped_g16_8192x8192x8192"] = time_grouped(16, 8192, 8192, 8192, dev, steps=20)
         configs["blockwise_8192x8192x8192"] = time_blockwise(8192, 8192, 8192, dev)
         configs["quantise_f32_8192x8192"] = time_quantiser(8192, 8192, torch.float32, dev)
         configs["quantise_bf16_8192x8192"] = time_quantiser(8192, 8192, torch.bfloat16, dev)
         configs["quantise_bf16_57344x8192"] = time_quantiser(57344, 8192, torch.bfloat16, dev, steps=20, copies=2)
-        if args.all_configs:
-            for (ln, lk) in [(10240, 8192), (8192, 8192), (57344, 8192), (8192, 28672)]:
-                for lm in (1, 32, 128, 1024, 4096):
-                    copies = max(2, min(8, int(600e6 // (ln * lk)) + 1))
-                    ls = make_device_inputs(lm, ln, lk, 0.02, False, dev, copies=copies)
-                    configs[f"c4_llama70b_{lm}x{ln}x{lk}"] = figures(lm, ln, lk, False, time_steps_graph(ls, 30, 3))
-                    del ls
-                    torch.cuda.empty_cache()
         line["configs"] = configs
 
     if not args.no_cpu_baseline:
-        xq, wq, xs, ws, _, _ = sets[0]
-        line["cpu_baseline"] = cpu_baseline(xq, wq, xs, ws)
+        line["cpu_baseline"] = cpu_baseline(head_sets[0], "M=N=K=8192")
 
     print(json.dumps(line))
 

@@ -165,7 +165,7 @@ int mi355x_fp8_rowwise_gemm_noalloc(const void* a, const void* b,
  * (grouped_gemm_fp8_rowwise(group_A, group_B, m_sizes, a_scale, b_scale)) and :426-455.
  *
  *   a        e4m3fn [M, K]                      b        e4m3fn [G*N, K]
- *   a_scale  f32 [M]                            b_scale  f32 [G*N], 16-byte aligned
+ *   a_scale  f32 [M]                            b_scale  f32 [G*N]
  *   m_sizes  int32 [G] in DEVICE memory         c        bf16 [M, N]
  *
  * The sizes are read by the kernel, not by the host (no synchronisation): negative sizes
@@ -209,7 +209,10 @@ int mi355x_fp8_blockwise_gemm(const void* a, const void* b,
  *   inv_scale[r] = 1 / scale[r]                                      (f32)
  * An f32 source is processed in f32. For a bf16 source every intermediate (scale, scaled
  * value, inverse scale) is rounded to bf16, which is how eager PyTorch evaluates the same
- * expression on a bf16 tensor. NaN inputs are not propagated (they quantise as +-448).
+ * expression on a bf16 tensor. Non-finite input behaves as in that program: a row holding a NaN
+ * comes out as NaN codes (0x7f / 0xff) with a NaN inverse scale; a row holding an infinity gets
+ * scale 0 and inverse scale infinity, its finite elements become (signed) zero and the
+ * infinities NaN.
  *
  *   x  [R, K] of `src_type`, row stride ldx (elements)     xq  e4m3fn [R, K], row stride ldq
  */

@@ -273,6 +273,26 @@ def test_padded_operands_and_output_canaries(gpu_device, variant, m):
     assert torch.all(c_buf[mask] == -77.0)
 
 
+@pytest.mark.parametrize("config", range(_lib.NUM_TILE_CONFIGS))
+def test_tiled_family_takes_unaligned_scale_and_bias_vectors(gpu_device, config):
+    # b_scale 4 bytes and bias 2 bytes into their allocations (a slice of a longer vector): full
+    # tiles then take the element-wise epilogue instead of being refused
+    m, n, k = 512, 512, 256
+    xq, wq, xs, ws, b = orc.make_inputs(m, n, k, 1.0, True)
+    want = orc.dequant_matmul(xq, wq, xs, ws, b)
+    dev = gpu_device
+    ws_buf = torch.zeros(n + 1, dtype=torch.float32, device=dev)
+    ws_buf[1:] = ws.to(dev)
+    bias_buf = torch.zeros(n + 1, dtype=torch.bfloat16, device=dev)
+    bias_buf[1:] = b.to(dev)
+    assert ws_buf[1:].data_ptr() % 16 == 4 and bias_buf[1:].data_ptr() % 8 == 2
+    out = ops.fp8_gemm_rowwise(xq.to(dev), wq.to(dev), xs.to(dev), ws_buf[1:], bias=bias_buf[1:],
+                               variant=_lib.tiled_variant(config, 1))
+    torch.cuda.synchronize()
+    torch.testing.assert_close(out.cpu(), want, rtol=RTOL, atol=ATOL)
+    _check_tight(out.cpu(), xq, wq, xs, ws, b)
+
+
 def test_bias_is_fused_before_the_single_rounding(gpu_device):
     a = torch.zeros(16, 16)
     a[0, 0] = 1.0
@@ -415,6 +435,35 @@ def test_quantiser_special_rows(gpu_device):
     xq, inv = ops.fp8_row_quantize(x.to(gpu_device))
     assert torch.equal(xq.cpu().view(torch.uint8), want_q.view(torch.uint8))
     assert torch.equal(inv.cpu().view(torch.int32), want_inv.view(torch.int32))
+
+
+@pytest.mark.parametrize("dtype,cols", [(torch.float32, 64), (torch.float32, 4100), (torch.float32, 61),
+                                        (torch.bfloat16, 64), (torch.bfloat16, 16400), (torch.bfloat16, 59)])
+def test_quantiser_non_finite_rows(gpu_device, dtype, cols):
+    # rows holding NaN or infinities come out as the PyTorch program leaves them (vector and scalar
+    # kernels, rows longer than the register cache): NaN codes wherever the oracle has NaN codes
+    # (the sign bit of a NaN is the platform's), every other code and every inverse scale bit for bit
+    x = orc.randn_f32(7, cols, 1.0, seed=cols).to(dtype)
+    x[1, 3] = float("nan")
+    x[2, 4] = float("inf")
+    x[2, cols - 1] = float("-inf")
+    x[3, 5] = float("-inf")
+    x[3, cols - 2] = float("nan")
+    x[5, cols // 2] = float("nan")
+    x[6] = 0.0
+    x[6, 1] = float("inf")
+    want_q, want_inv = orc.fp8_row_quantize(x)
+    xq, inv = ops.fp8_row_quantize(x.to(gpu_device))
+    torch.cuda.synchronize()
+    got, want = xq.cpu().view(torch.uint8).numpy(), want_q.view(torch.uint8).numpy()
+    want_nan = (want & 0x7F) == 0x7F
+    assert want_nan[1].all() and want_nan[3].all() and want_nan[5].all() and want_nan[2].sum() == 2 and want_nan[6].sum() == 1
+    assert np.array_equal((got & 0x7F) == 0x7F, want_nan)
+    assert np.array_equal(got[~want_nan], want[~want_nan])
+    gi, wi = inv.cpu().numpy(), want_inv.numpy()
+    assert np.array_equal(np.isnan(gi), np.isnan(wi))
+    assert np.array_equal(gi[~np.isnan(wi)].view(np.uint32), wi[~np.isnan(wi)].view(np.uint32))
+    assert np.isinf(gi[2]) and np.isinf(gi[6])
 
 
 def test_quantise_then_gemm_end_to_end(gpu_device):

@@ -425,6 +425,11 @@ def test_cuda_time_groups_kernels_between_flush_fills():
     ]
     assert split_calls(reversed(events)) == pytest.approx([0.026, 0.027, 0.014])
     assert split_calls([]) == []
+    # a backend that zero-fills its own bf16 output inside the call is not taken for the flush
+    own_fill = fill.replace("FillFunctor<int>", "FillFunctor<c10::BFloat16>")
+    events = [(10.0, 70.0, fill), (90.0, 3.0, own_fill), (95.0, 20.0, "grouped gemm"),
+              (120.0, 70.0, fill), (200.0, 3.0, own_fill), (205.0, 21.0, "grouped gemm")]
+    assert split_calls(events) == pytest.approx([0.023, 0.024])
 
 
 def test_cuda_time_metric_needs_a_gpu_backend():

@@ -88,3 +88,32 @@ def test_bf16_source_runs_in_bf16():
     scale = (448.0 / x.abs().max(dim=1).values)
     assert scale.dtype == torch.bfloat16
     assert torch.equal(inv, scale.reciprocal().float())
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_non_finite_rows_follow_the_torch_program(dtype):
+    # what operator.py:136-145 does with NaN and infinities, fixed by torch.max / clamp / the fp8
+    # cast: a NaN poisons its row (NaN maximum -> NaN scale -> every code NaN, NaN inverse scale);
+    # an infinity gives scale 1/inf * 448 = 0 (finite elements -> signed zero, inf * 0 -> NaN) and
+    # inverse scale +inf. Other rows are untouched. The sign bit of a NaN code is whatever the
+    # platform's arithmetic leaves in the NaN, so NaN codes are compared as NaN only.
+    x = orc.randn_f32(5, 64, 1.0, seed=77).to(dtype)
+    x[1, 3] = float("nan")
+    x[2, 4] = float("inf")
+    x[2, 9] = float("-inf")
+    x[3, 5] = float("-inf")
+    x[3, 6] = float("nan")
+    xq, inv = orc.fp8_row_quantize(x)
+    codes = _codes(xq)
+    is_nan = (codes & 0x7F) == 0x7F
+    assert is_nan[1].all() and is_nan[3].all()
+    assert np.isnan(inv[1].item()) and np.isnan(inv[3].item())
+    assert inv[2].item() == float("inf")
+    inf_at = torch.isinf(x[2].float()).numpy()
+    assert is_nan[2][inf_at].all()
+    want_zero = np.where(np.signbit(x[2].float().numpy()[~inf_at]), 0x80, 0x00)
+    assert np.array_equal(codes[2][~inf_at], want_zero)
+    for r in (0, 4):
+        alone_q, alone_inv = orc.fp8_row_quantize(x[r:r + 1].clone())
+        assert np.array_equal(codes[r], _codes(alone_q)[0]) and inv[r] == alone_inv[0]
+        assert not is_nan[r].any()

@@ -821,8 +821,10 @@ void gemm_tiled_kernel(GemmParams p) {
         // sb already names the next step's stage; the one before it held this tile's last step
         uint8_t* free_b = lds + LDS_B0 + ((sb + kStagesB - 1) % kStagesB) * STAGE_B;
         const bool interior = (loc.m0 + BM <= loc.m_end) && (loc.n0 + BN <= p.N);
-        // b_scale is read 16 bytes at a time on this path: a group's slice must start aligned
+        // the vector epilogue stores 16 bytes of C and reads b_scale 16 and bias 8 bytes at a time
+        // (a group's slice of b_scale must start aligned too); anything else takes the scalar one
         const uintptr_t bits = reinterpret_cast<uintptr_t>(p.c) | (uintptr_t)(p.ldc * 2) |
+                               reinterpret_cast<uintptr_t>(p.b_scale) | (reinterpret_cast<uintptr_t>(p.bias) << 1) |
                                (GROUPED ? (uintptr_t)(p.N * 4) : 0);
         if (interior && (bits & 15) == 0) epilogue(loc, std::true_type{}, free_b);
         else epilogue(loc, std::false_type{}, free_b);
@@ -1317,6 +1319,33 @@ struct SrcTraits<uint16_t> {
   static __device__ __forceinline__ float round(float v) { return bf16_to_f32(f32_to_bf16_rne(v)); }
 };
 
+// max(a, b) that returns NaN when either operand is NaN (torch.max does; fmaxf drops the NaN).
+// One gfx950 instruction (v_maximum3_f32).
+__device__ __forceinline__ float max_keep_nan(float a, float b) { return __builtin_elementwise_maximum(a, b); }
+
+// The row's quantisation scale from its absolute maximum, as eager PyTorch computes it:
+// `448.0 / clamp(amax, 1e-12)` evaluates as reciprocal * 448, and clamp keeps a NaN (so a row
+// holding a NaN gets a NaN scale, a row holding an infinity the scale 0).
+template <typename SrcT>
+__device__ __forceinline__ float row_scale(float amax) {
+  using T = SrcTraits<SrcT>;
+  const float floor_ = T::round(1e-12f);
+  const float clamped = amax < floor_ ? floor_ : amax;  // false for NaN: it stays
+  const float recip = T::round(1.0f / clamped);
+  return T::round(recip * 448.0f);
+}
+
+// One element the way the PyTorch program treats it, NaN included: scale, clamp to +-448 (a NaN
+// passes the clamp), round to e4m3fn with the integer encoder (NaN -> 0x7f with the sign kept).
+template <typename SrcT>
+__device__ __forceinline__ uint8_t quantize_one(float x, float scale) {
+  using T = SrcTraits<SrcT>;
+  float v = T::round(x * scale);
+  v = v < -448.0f ? -448.0f : v;
+  v = v > 448.0f ? 448.0f : v;
+  return f32_to_e4m3fn_rne(v);
+}
+
 template <typename SrcT>
 __global__ __launch_bounds__(256) void quantize_rows_kernel(const SrcT* x, uint8_t* xq,
                                                             float* inv_scale, int K, long ldx,
@@ -1328,22 +1357,16 @@ __global__ __launch_bounds__(256) void quantize_rows_kernel(const SrcT* x, uint8
   uint8_t* qr = xq + row * ldq;
 
   float amax = 0.0f;
-  for (int k = threadIdx.x; k < K; k += 256) amax = fmaxf(amax, fabsf(T::load(xr + k)));
+  for (int k = threadIdx.x; k < K; k += 256) amax = max_keep_nan(amax, fabsf(T::load(xr + k)));
 #pragma unroll
-  for (int o = 32; o > 0; o >>= 1) amax = fmaxf(amax, __shfl_xor(amax, o));
+  for (int o = 32; o > 0; o >>= 1) amax = max_keep_nan(amax, __shfl_xor(amax, o));
   if ((threadIdx.x & 63) == 0) wave_max[threadIdx.x >> 6] = amax;
   __syncthreads();
-  amax = fmaxf(fmaxf(wave_max[0], wave_max[1]), fmaxf(wave_max[2], wave_max[3]));
+  amax = max_keep_nan(max_keep_nan(wave_max[0], wave_max[1]), max_keep_nan(wave_max[2], wave_max[3]));
 
-  // `448.0 / tensor` in the PyTorch program this replaces evaluates as reciprocal * 448
-  const float recip = T::round(1.0f / fmaxf(amax, T::round(1e-12f)));
-  const float scale = T::round(recip * 448.0f);
+  const float scale = row_scale<SrcT>(amax);
   if (threadIdx.x == 0) inv_scale[row] = T::round(1.0f / scale);
-  for (int k = threadIdx.x; k < K; k += 256) {
-    float v = T::round(T::load(xr + k) * scale);
-    v = fminf(fmaxf(v, -448.0f), 448.0f);
-    qr[k] = f32_to_e4m3fn_rne(v);
-  }
+  for (int k = threadIdx.x; k < K; k += 256) qr[k] = quantize_one<SrcT>(T::load(xr + k), scale);
 }
 
 // Vector form of the quantiser for 16-byte aligned rows: one workgroup per row, every lane
@@ -1394,7 +1417,7 @@ __global__ __launch_bounds__(THREADS) void quantize_rows_vec_kernel(const SrcT* 
     float f[EPV];
     V::unpack(c, f);
 #pragma unroll
-    for (int e = 0; e < EPV; ++e) amax = fmaxf(amax, fabsf(f[e]));
+    for (int e = 0; e < EPV; ++e) amax = max_keep_nan(amax, fabsf(f[e]));
   };
 #pragma unroll
   for (int i = 0; i < CACHE; ++i) {
@@ -1406,15 +1429,22 @@ __global__ __launch_bounds__(THREADS) void quantize_rows_vec_kernel(const SrcT* 
   for (int i = 0; i < CACHE; ++i) fold(cache[i]);
   for (int c = tid + THREADS * CACHE; c < nchunks; c += THREADS) fold(xr[c]);
 #pragma unroll
-  for (int o = 32; o > 0; o >>= 1) amax = fmaxf(amax, __shfl_xor(amax, o));
+  for (int o = 32; o > 0; o >>= 1) amax = max_keep_nan(amax, __shfl_xor(amax, o));
   if ((tid & 63) == 0) wave_max[tid >> 6] = amax;
   __syncthreads();
 #pragma unroll
-  for (int w = 0; w < THREADS / 64; ++w) amax = fmaxf(amax, wave_max[w]);
+  for (int w = 0; w < THREADS / 64; ++w) amax = max_keep_nan(amax, wave_max[w]);
 
-  const float recip = T::round(1.0f / fmaxf(amax, T::round(1e-12f)));
-  const float scale = T::round(recip * 448.0f);
+  const float scale = row_scale<SrcT>(amax);
   if (tid == 0) inv_scale[row] = T::round(1.0f / scale);
+  // A row that holds a NaN or an infinity (the whole workgroup sees the same amax) takes the
+  // element-by-element route, whose clamp and encoder carry NaN through as PyTorch does; the
+  // pack-convert route below is for finite rows.
+  if (!(amax < __builtin_inff())) {
+    const SrcT* xs = x + row * ldx;
+    for (int k = tid; k < K; k += THREADS) qr[k] = quantize_one<SrcT>(T::load(xs + k), scale);
+    return;
+  }
 
   auto convert = [&](const v4i& src, uint32_t (&out)[EPV / 4]) {
     float f[EPV];
@@ -1611,11 +1641,32 @@ inline TiledPlan plan_from_variant(int64_t M, int64_t N, int64_t K, int variant,
 // Raises a kernel's dynamic-LDS limit once per device (the attribute belongs to the device's
 // copy of the code object). Idempotent, so a race between threads is harmless.
 constexpr int kMaxDevices = 64;
+// The tile walk, the grid sizes and the cost tables are written for the whole part: 256 CUs in 8
+// XCDs. A device that reports another CU count (a partitioned mode, another product) would be
+// scheduled wrongly without any error, so it is turned away here, once per device.
+int check_device_shape(int dev) {
+  static std::atomic<int> seen[kMaxDevices];  // 0 unknown, 1 fits, -1 does not
+  const bool tracked = dev >= 0 && dev < kMaxDevices;
+  int state = tracked ? seen[dev].load(std::memory_order_relaxed) : 0;
+  int cus = 0;
+  if (state == 0) {
+    const hipError_t e = hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev);
+    if (e != hipSuccess) return fail(MI355X_FP8_ELAUNCH, "hipDeviceGetAttribute: %s", hipGetErrorString(e));
+    state = cus == kNumCu ? 1 : -1;
+    if (tracked) seen[dev].store(state, std::memory_order_relaxed);
+  }
+  if (state < 0)
+    return fail(MI355X_FP8_ENOTSUP, "device %d does not report the %d compute units these kernels are scheduled for "
+                "(a partitioned mode or another part)", dev, kNumCu);
+  return MI355X_FP8_OK;
+}
+
 int raise_lds_limit(const void* kernel, size_t lds_bytes, bool (&done)[kMaxDevices]) {
   int dev = 0;
   hipError_t e = hipGetDevice(&dev);
   if (e != hipSuccess) return fail(MI355X_FP8_ELAUNCH, "hipGetDevice: %s", hipGetErrorString(e));
   if (dev >= 0 && dev < kMaxDevices && done[dev]) return MI355X_FP8_OK;
+  if (const int st = check_device_shape(dev)) return st;
   e = hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
   if (e != hipSuccess) return fail(MI355X_FP8_ELAUNCH, "hipFuncSetAttribute: %s", hipGetErrorString(e));
   if (dev >= 0 && dev < kMaxDevices) done[dev] = true;
@@ -1834,9 +1885,6 @@ int mi355x_fp8_rowwise_gemm_ex(const void* a, const void* b, const float* a_scal
 
   switch (variant) {
     case MI355X_FP8_VARIANT_TILED:
-      // b_scale is read 16 bytes at a time on full tiles
-      if (reinterpret_cast<uintptr_t>(b_scale) & 15 || (bias && (reinterpret_cast<uintptr_t>(bias) & 7)))
-        return fail(MI355X_FP8_ENOTSUP, "tiled variant needs b_scale 16-byte and bias 8-byte aligned");
       {
         // A caller that brought no (or too little) workspace gets the best plan that needs none,
         // unless it asked for a split factor by name.
@@ -1918,9 +1966,9 @@ int mi355x_fp8_rowwise_grouped_gemm(const void* a, const void* b, const float* a
   if (lda % 16 || ldb % 16) return fail(MI355X_FP8_ENOTSUP, "lda and ldb must be multiples of 16");
   if ((reinterpret_cast<uintptr_t>(a) & 15) || (reinterpret_cast<uintptr_t>(b) & 15))
     return fail(MI355X_FP8_ENOTSUP, "a and b must be 16-byte aligned");
-  if ((reinterpret_cast<uintptr_t>(a_scale) & 3) || (reinterpret_cast<uintptr_t>(b_scale) & 15) ||
+  if ((reinterpret_cast<uintptr_t>(a_scale) & 3) || (reinterpret_cast<uintptr_t>(b_scale) & 3) ||
       (reinterpret_cast<uintptr_t>(c) & 1) || (reinterpret_cast<uintptr_t>(m_sizes) & 3))
-    return fail(MI355X_FP8_EINVAL, "misaligned scale, size or output pointer (b_scale needs 16 bytes)");
+    return fail(MI355X_FP8_EINVAL, "misaligned scale, size or output pointer");
   if (lda * 256 > (int64_t)UINT32_MAX || ldb * 256 > (int64_t)UINT32_MAX)
     return fail(MI355X_FP8_ENOTSUP, "leading dimension too large");
   if (tile_config < -1 || tile_config >= kNumGroupedTileConfigs)

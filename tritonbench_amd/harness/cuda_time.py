@@ -3,8 +3,8 @@
 The upstream metric (tritonbench/components/do_bench/cuda_time.py:12-110) profiles repeated
 `cache.zero_(); fn()` pairs with the PyTorch profiler and adds up, per call, the durations of
 every device kernel except the cache-clearing fill, which it recognises by its full CUDA
-kernel name. Here the fill is recognised by the functor it instantiates (`FillFunctor`, the
-same on ROCm and CUDA builds, whatever the rest of the template spells), the flush buffer is
+kernel name. Here the fill is recognised by the functor it instantiates (`FillFunctor<int>`: the
+flush buffer is int32; the same on ROCm and CUDA builds, whatever the rest of the template spells), the flush buffer is
 twice the MI355X memory-side cache (upstream's 256 MB equals that cache and leaves operands
 in it), and a call's kernels are the ones between two fills in start order, so backends that
 launch a different number of kernels per call (a split-K plan launches two) need no
@@ -13,7 +13,9 @@ from typing import Callable, List
 
 from .latency import FLUSH_BYTES, Latency
 
-FLUSH_KERNEL_MARK = "FillFunctor"
+# the flush buffer is int32, so its fill instantiates FillFunctor<int>: a backend whose callable
+# zero-fills its own (bf16, float, ...) output inside the call is not mistaken for the flush
+FLUSH_KERNEL_MARK = "FillFunctor<int>"
 
 
 def split_calls(events) -> List[float]:

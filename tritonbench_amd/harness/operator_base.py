@@ -33,6 +33,7 @@ import tabulate
 import torch
 
 from . import registry as R
+from . import rocprof
 from .latency import Latency, do_bench_wrapper
 
 logger = logging.getLogger(__name__)
@@ -345,7 +346,9 @@ class BenchmarkOperator(metaclass=_PostInit):
                 ref = ref.to(out.device)
             torch.testing.assert_close(out, ref, rtol=getattr(self.tb_args, "rtol", None), atol=getattr(self.tb_args, "atol", None))
             return True
-        except Exception:
+        except Exception as e:
+            logger.warning("accuracy of %s against %s failed: %s", getattr(fn, "_name", fn),
+                           getattr(baseline_fn, "_name", baseline_fn), str(e).strip().splitlines()[0] if str(e).strip() else repr(e))
             return False
 
     def tflops(self, fn_name: str, example_inputs: Any, metrics: BenchmarkOperatorMetrics) -> Optional[float]:
@@ -396,6 +399,15 @@ class BenchmarkOperator(metaclass=_PostInit):
                 from .cuda_time import do_bench_cuda_time
 
                 rec.cuda_time = do_bench_cuda_time(fn, warmup, rep)
+            if want & {"rocprof", "rocprof_us", rocprof.IN_TASK_METRIC}:
+                if backend_device == "cpu" or not torch.cuda.is_available():
+                    raise NotImplementedError("rocprof needs a GPU backend")
+                if rocprof.IN_TASK_METRIC in want:  # this process IS the profiled child
+                    rec.extra_metrics[rocprof.IN_TASK_METRIC] = rocprof.run_in_task(fn)
+                else:
+                    rows = rocprof.profile_backend(self.name, fn_name, input_id, self.tb_args, self._raw_extra_args)
+                    rec.extra_metrics["rocprof"] = rocprof.format_rows(rows)
+                    rec.extra_metrics["rocprof_us"] = sum(r["us_per_call"] for r in rows)
             if "gpu_peak_mem" in want and self.device == "cuda":
                 torch.cuda.reset_peak_memory_stats()
                 fn()

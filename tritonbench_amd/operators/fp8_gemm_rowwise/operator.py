@@ -14,6 +14,7 @@ Backends here:
                        the variant upstream leaves commented out at :237-246
 """
 import argparse
+import logging
 from typing import Any, Callable, Generator, List, Optional, Tuple
 
 import torch
@@ -26,6 +27,8 @@ from tritonbench_amd.harness import (
     register_metric,
     register_x_val,
 )
+
+logger = logging.getLogger(__name__)
 
 FP8_DTYPE = torch.float8_e4m3fn
 E4M3_MAX_POS: float = torch.finfo(FP8_DTYPE).max
@@ -207,7 +210,9 @@ class Operator(BenchmarkOperator):
             out, ref = fn(), baseline_fn()
             torch.testing.assert_close(out.cpu(), ref.cpu(), rtol=rtol, atol=atol)
             return True
-        except Exception:
+        except Exception as e:  # the cell reads False; the reason goes to the log, not into the void
+            logger.warning("accuracy of %s against %s failed: %s", getattr(fn, "_name", fn),
+                           getattr(baseline_fn, "_name", baseline_fn), str(e).strip().splitlines()[0] if str(e).strip() else repr(e))
             return False
 
     @register_x_val(label="(M, N, K)")
