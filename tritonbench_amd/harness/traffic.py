@@ -6,7 +6,7 @@ JSON summary bench.py reports as `roofline.traffic`.
     python -m tritonbench_amd.harness.traffic --dir <dir> --kernel "gemm_tiled_kernel<256, 256" --out profiles/tiled_8192cubed_traffic.json
 
 Both counters read KiB per dispatch; each is scaled by what it reads for the copy kernel of
-known size that bench.py launches in the same run (an elementwise multiply of a 256 MiB tensor).
+known size that bench.py launches in the same run (an elementwise negation of a 256 MiB tensor).
 The summary records the hash of the kernel source it was measured on; bench.py marks a summary
 whose hash differs from the present source as stale.
 """
