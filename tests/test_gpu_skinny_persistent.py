@@ -1,4 +1,5 @@
-"""Parity of the persistent skinny kernel (M <= 16, N % 16 == 0, K in {2048, 4096, 6144, 8192})
+"""Parity of the persistent skinny kernel (N % 16 == 0; M <= 16 with K in {2048, 4096, 6144, 8192},
+M <= 32 with K = 4096: two 16-row blocks of A resident in registers)
 with the CPU oracle, and against the one-tile-per-workgroup kernel it replaces on those shapes.
 Both are reached through the C ABI with the skinny family pinned. Needs an MI355X."""
 import numpy as np
@@ -55,13 +56,17 @@ SHAPES = [
     (1, 16, 2048, False), (16, 16, 8192, True), (7, 48, 4096, True), (16, 4096, 2048, False),
     (9, 4112, 6144, True), (16, 8192, 4096, False), (3, 8208, 2048, True), (16, 10240, 2048, True),
     (13, 2064, 8192, False), (16, 12304, 2048, False),
+    # two blocks of A (M = 17..32, K = 4096): last block full / one row / ragged
+    (17, 16, 4096, True), (32, 8192, 4096, False), (25, 4112, 4096, True), (32, 10240, 4096, False),
+    (20, 2064, 4096, True), (31, 12304, 4096, False),
 ]
 
 
 @pytest.mark.parametrize("m,n,k,bias", SHAPES)
 def test_persistent_kernel_against_oracle(gpu_device, m, n, k, bias):
     print(f"case m={m} n={n} k={k} bias={bias}", flush=True)
-    assert ops.select_variant(m, n, k) == _lib.VARIANT_SKINNY  # what the automatic choice runs too
+    if m <= 16:
+        assert ops.select_variant(m, n, k) == _lib.VARIANT_SKINNY  # what the automatic choice runs too
     xq, wq, xs, ws, b = orc.make_inputs(m, n, k, 1.0, bias)
     want = orc.dequant_matmul(xq, wq, xs, ws, b)
     out = _run(gpu_device, xq, wq, xs, ws, b, PERSISTENT)
@@ -73,7 +78,7 @@ def test_persistent_kernel_against_oracle(gpu_device, m, n, k, bias):
     _check_tight(other, xq, wq, xs, ws, b)
 
 
-@pytest.mark.parametrize("m,k", [(16, 2048), (5, 8192)])
+@pytest.mark.parametrize("m,k", [(16, 2048), (5, 8192), (32, 4096), (19, 4096)])
 def test_exact_integer_case_is_bit_exact(gpu_device, m, k):
     # small integers, unit scales: every partial sum stays below 2^24, so fp32 summation is
     # exact in any order and both kernels must reproduce the float64 result bit for bit

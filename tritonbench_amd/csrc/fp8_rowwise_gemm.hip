@@ -162,19 +162,19 @@ constexpr int kDefaultDist = 2;  // steps a load runs ahead of its use; A ring =
 
 __device__ __forceinline__ int swz128(int row) { return (row >> 1) & 7; }
 
-// STREAM marks the lines as used once (the instruction's `nt` bit): they leave the L2 early
-// instead of pushing out lines other workgroups will ask for again.
-template <bool STREAM = false>
-__device__ __forceinline__ void load_chunk_to_lds(const uint8_t* gsrc, uint8_t* lds_wave_base) {
-  // Each lane fetches 16 bytes; the hardware deposits lane i's bytes at lds_wave_base + 16*i.
-  __builtin_amdgcn_global_load_lds(
-      (const __attribute__((address_space(1))) void*)gsrc,
-      (__attribute__((address_space(3))) void*)lds_wave_base, 16, 0, STREAM ? 2 : 0);
+// One wave-wide load of 16 bytes per lane from a buffer straight into LDS: lane i's bytes land at
+// lds_wave_base + 16*i. The address is the descriptor's base + lane_off + wave_off, range-checked
+// against the descriptor's extent (bytes past it arrive as zeros). STREAM marks the lines as used
+// once (the instruction's `nt` bit): they leave the L2 early instead of pushing out lines other
+// workgroups will ask for again.
+template <bool STREAM>
+__device__ __forceinline__ void load_chunk_to_lds(__amdgpu_buffer_rsrc_t rsrc, uint8_t* lds_wave_base,
+                                                  uint32_t lane_off, uint32_t wave_off) {
+#if defined(__HIP_DEVICE_COMPILE__)  // (the host pass does not know the builtin)
+  __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, (__attribute__((address_space(3))) void*)lds_wave_base, 16,
+                                           (int)lane_off, (int)wave_off, 0, STREAM ? 2 : 0);
+#endif
 }
-
-// Source of the chunks that lie past K in the last, partial K step: the operands there must
-// read as zeros (whatever follows a row in memory could decode to NaN).
-__device__ const v4i kZeroChunk = {0, 0, 0, 0};
 
 // Waits until at most VM of this wave's global loads and none of its LDS operations are
 // outstanding, then joins the workgroup barrier. Written with the s_waitcnt builtin (not
@@ -358,111 +358,120 @@ void gemm_tiled_kernel(GemmParams p) {
     c.left = c.kt_end - c.kt_begin;
     c.kt = c.kt_begin + (STREAM_B && p.splits <= 2 ? (loc.n0 / BN) % c.left : 0);
   };
-  const uint8_t* l_a = nullptr;
-  const uint8_t* l_b = nullptr;
-  // Source address of a lane's 16 bytes in the i-th 8-row group (grp = wave + NW*i) a wave fetches:
-  // tile base + K offset + a 32-bit lane offset, row*ld + chunk, with rows past the matrix edge
-  // redirected to the last valid row (they are read but never stored, so every load stays in
-  // bounds without predication). Two forms:
-  //  * one offset register per group (small tiles);
-  //  * 256x256 tile, where registers are short (16 of these per lane used to end up in scratch,
-  //    and every reload there waits for all loads in flight): 8*grp*ld goes into the scalar
-  //    base and the lane part, ld_row*ld + chunk, is one register for all groups (the chunk
-  //    depends on the group's parity only, which a wave's groups share). Only the group that
-  //    holds the edge needs its own lane part (rows clamped inside the group); groups behind it
-  //    are sent there too. Costs a few scalar instructions and a select per load.
+  // Source of the loads: one buffer descriptor per operand and tile, base = the tile's first row,
+  // extent = its valid rows (the hardware returns zeros for anything past the extent, so rows past
+  // the matrix edge need neither clamping nor predication: they read as zeros and are never
+  // stored). A lane's 16 bytes in the i-th 8-row group a wave fetches (grp = wave + NW*i) lie at
+  //   lane part (vector register, the same for every group, step and tile: ld_row*ld + chunk,
+  //              the chunk swizzle depends on the group's parity only, which a wave's groups share)
+  // + scalar part (K offset + 8*grp*ld, one scalar add per load).
+  // The range check adds the two before it compares, so the sum must stay below 2^32: the host
+  // admits leading dimensions up to 2^31 / 256.
   static_assert(NW % 2 == 0, "all groups of a wave must share their parity");
-  constexpr bool SHARED_OFFSETS = BM * BN >= 256 * 256;
-  constexpr int MAX_GROUPS = A_GROUPS > B_GROUPS ? A_GROUPS : B_GROUPS;
-  struct OperandOffsets {
-    uint32_t per_group[SHARED_OFFSETS ? 1 : MAX_GROUPS];
-    uint32_t full, edge;  // shared form: lane part of whole groups / of the group with the edge
-    int last_group;       // shared form: the group that holds the last valid row
-    uint32_t ld;
+  struct OperandSrc {
+    const uint8_t* base;
+    uint32_t extent;                  // bytes from base that may be read
+    uint32_t wave_off, group_stride;  // 8*wave*ld and 8*NW*ld
   };
-  // 24-bit multiplies (row < 2^8, leading dimension < 2^24 by the host's check): one instruction
-  // and a 32-bit result, where the full multiply leaves a 64-bit register pair
-  auto make_offsets = [&](int rows_valid, long ld, int groups) -> OperandOffsets {
-    const int last_row = max(rows_valid - 1, 0);
-    OperandOffsets o = {{0}, 0, 0, 0, (uint32_t)ld};
-    if (SHARED_OFFSETS) {
-      const uint32_t chunk = ld_chunk_off(wave);
-      o.full = __umul24((uint32_t)ld_row, (uint32_t)ld) + chunk;
-      o.edge = __umul24((uint32_t)min(ld_row, last_row & 7), (uint32_t)ld) + chunk;
-      o.last_group = last_row >> 3;
-    } else {
-#pragma unroll
-      for (int i = 0; i < MAX_GROUPS; ++i) {
-        const int grp = wave + NW * i;
-        if (i < groups) o.per_group[i] = __umul24((uint32_t)min(grp * 8 + ld_row, last_row), (uint32_t)ld) + ld_chunk_off(grp);
-      }
-    }
+  constexpr int kRsrcFlags = 0x00020000;  // raw buffer, 32-bit data format: plain byte addressing with range check
+  auto make_src = [&](const uint8_t* base, int rows_valid, int rows_tile, long ld) -> OperandSrc {
+    // (a tile always starts on a valid row, so rows_valid >= 1; clamping at zero as well would turn
+    // the pair into a three-operand median, which exists as a vector instruction only and would
+    // pull the descriptor out of the scalar registers)
+    const uint32_t extent = (uint32_t)min(rows_valid, rows_tile) * (uint32_t)ld;
+    OperandSrc o;
+    o.base = base;
+    o.extent = extent;
+    o.wave_off = 8u * (uint32_t)wave * (uint32_t)ld;
+    o.group_stride = 8u * NW * (uint32_t)ld;
     return o;
   };
-  auto group_src = [&](const uint8_t* g, const OperandOffsets& o, int i) -> const uint8_t* {
-    if (!SHARED_OFFSETS) return g + o.per_group[i];
-    const int grp = wave + NW * i;
-    const uint32_t rows_off = (uint32_t)min(grp, o.last_group) * 8u * o.ld;  // < 2^32 by the same check
-    return g + rows_off + (grp < o.last_group ? o.full : o.edge);
-  };
-  OperandOffsets a_off = {{0}, 0, 0, 0, 0}, b_off = {{0}, 0, 0, 0, 0};
+  // 24-bit multiplies (row < 8, leading dimension < 2^24 by the host's check)
+  const uint32_t lane_chunk = (uint32_t)ld_chunk_off(wave);
+  const uint32_t a_lane = __umul24((uint32_t)ld_row, (uint32_t)p.lda) + lane_chunk;
+  const uint32_t b_lane = __umul24((uint32_t)ld_row, (uint32_t)p.ldb) + lane_chunk;
+  // K tail (KTAIL kernels only): in the partial last step, lanes whose chunk lies at or past K
+  // must fetch zeros (whatever follows a row in memory could decode to NaN): their lane part is
+  // pushed past every extent for that step. A lane's logical chunk is the same for all its
+  // groups.
+  const bool tail_chunk_ok = ((ld_pc ^ swz128(wave * 8 + ld_row)) * kChunk) < k_tail;
+  constexpr uint32_t kPastExtent = 0x80000000u;  // extents and scalar parts stay below 2^31
+  const uint32_t a_lane_tail = tail_chunk_ok ? a_lane : kPastExtent;
+  const uint32_t b_lane_tail = tail_chunk_ok ? b_lane : kPastExtent;
+  OperandSrc a_src = {nullptr, 0, 0, 0}, b_src = {nullptr, 0, 0, 0};
   auto setup_a = [&](int li) {
     const TileLoc loc = locate(walk_a, li);
     start_cursor(ca, li, loc);
-    l_a = p.a + (size_t)loc.m0 * p.lda;
-    a_off = make_offsets(loc.m_end - loc.m0, p.lda, A_GROUPS);
+    a_src = make_src(p.a + (size_t)loc.m0 * p.lda, loc.m_end - loc.m0, BM, p.lda);
   };
   auto setup_b = [&](int li) {
     const TileLoc loc = locate(walk_b, li);
     start_cursor(cb, li, loc);
-    l_b = p.b + ((size_t)loc.group * p.N + loc.n0) * p.ldb;
-    b_off = make_offsets(p.N - loc.n0, p.ldb, B_GROUPS);
+    b_src = make_src(p.b + ((size_t)loc.group * p.N + loc.n0) * p.ldb, p.N - loc.n0, BN, p.ldb);
   };
-  // Issues one operand's loads for its cursor's step into stage (issued % STAGES). Past the
+  // i-th group of one operand's step kt into the stage at sbase
+  // (step_off: K offset of the step + the wave's first group, prepared once per step)
+  auto load_group = [&](auto stream_tag, const OperandSrc& src, uint32_t lane_off, uint32_t step_off, int i, uint8_t* sbase) {
+    // (the descriptor is put together from its scalar parts here: one scalar instruction)
+    const __amdgpu_buffer_rsrc_t rsrc =
+        __builtin_amdgcn_make_buffer_rsrc(const_cast<uint8_t*>(src.base), 0, (int)src.extent, kRsrcFlags);
+    load_chunk_to_lds<decltype(stream_tag)::value>(rsrc, sbase + (wave + NW * i) * 1024, lane_off,
+                                                   step_off + (uint32_t)i * src.group_stride);
+  };
+  auto lane_part = [&](uint32_t whole, uint32_t tail, int kt) -> uint32_t {
+    return KTAIL && kt >= k_full ? tail : whole;
+  };
+  // Ring positions the next loads of A and of B go to (= issued % stages, kept as counters that wrap).
+  int fill_a = 0, fill_b = 0;
+  auto next_fill_a = [&]() { fill_a = (fill_a + 1 == kStagesA) ? 0 : fill_a + 1; };
+  auto next_fill_b = [&]() { fill_b = (fill_b + 1 == kStagesB) ? 0 : fill_b + 1; };
+  // Issues one operand's loads for its cursor's step into the next stage of its ring. Past the
   // last step it re-issues the last one into a stage nobody reads again, which keeps the
   // path free of branches.
-  // K tail (KTAIL kernels only): in the partial last step, lanes whose chunk lies at or past
-  // K fetch the zero chunk instead. A lane's logical chunk is the same for all its groups
-  // (the swizzle key depends on the group's parity only, and a wave's groups are NW apart).
-  const bool tail_chunk_ok = ((ld_pc ^ swz128(wave * 8 + ld_row)) * kChunk) < k_tail;
-  auto chunk_src = [&](const uint8_t* g, const OperandOffsets& o, int i, bool real) -> const uint8_t* {
-    if (!KTAIL) return group_src(g, o, i);
-    return real ? group_src(g, o, i) : reinterpret_cast<const uint8_t*>(&kZeroChunk);
-  };
-  auto issue = [&](auto stream_tag, const uint8_t* gbase, const OperandOffsets& off, int groups, int kt, uint8_t* sbase) {
-    const uint8_t* g = gbase + (size_t)kt * kStepK;
-    const bool real = !KTAIL || kt < k_full || tail_chunk_ok;
-#pragma unroll
-    for (int i = 0; i < MAX_GROUPS; ++i)
-      if (i < groups)
-        load_chunk_to_lds<decltype(stream_tag)::value>(chunk_src(g, off, i, real), sbase + (wave + NW * i) * 1024);
-  };
   auto issue_a = [&]() {
-    issue(std::false_type{}, l_a, a_off, A_GROUPS, ca.kt, lds + (ca.issued % kStagesA) * STAGE_A);
+    const uint32_t lo = lane_part(a_lane, a_lane_tail, ca.kt);
+#pragma unroll
+    for (int i = 0; i < A_GROUPS; ++i)
+      load_group(std::false_type{}, a_src, lo, (uint32_t)ca.kt * kStepK + a_src.wave_off, i, lds + fill_a * STAGE_A);
+    next_fill_a();
     ++ca.issued;
   };
   auto issue_b = [&]() {
-    issue(std::integral_constant<bool, STREAM_B>{}, l_b, b_off, B_GROUPS, cb.kt,
-          lds + LDS_B0 + (cb.issued % kStagesB) * STAGE_B);
+    const uint32_t lo = lane_part(b_lane, b_lane_tail, cb.kt);
+#pragma unroll
+    for (int i = 0; i < B_GROUPS; ++i)
+      load_group(std::integral_constant<bool, STREAM_B>{}, b_src, lo, (uint32_t)cb.kt * kStepK + b_src.wave_off, i,
+                 lds + LDS_B0 + fill_b * STAGE_B);
+    next_fill_b();
     ++cb.issued;
   };
-  auto advance_a = [&]() {
-    if (ca.issued >= total_steps) return;  // stay on the last step
-    if (--ca.left == 0) {
-      ca.item += walk.slots;
-      setup_a(ca.item);
-    } else if (++ca.kt == ca.kt_end) {
-      ca.kt = ca.kt_begin;
+  // Moves a load cursor to its next step. PLAIN: the caller knows that the next step belongs to the
+  // same work item (true for all but the last DIST + 1 steps of an item): no branch, no tile set-up.
+  auto advance_a = [&](auto plain_tag) {
+    if (!decltype(plain_tag)::value) {
+      if (ca.issued >= total_steps) return;  // stay on the last step
+      if (--ca.left == 0) {
+        ca.item += walk.slots;
+        setup_a(ca.item);
+        return;
+      }
+    } else {
+      --ca.left;
     }
+    ca.kt = (ca.kt + 1 == ca.kt_end) ? ca.kt_begin : ca.kt + 1;
   };
-  auto advance_b = [&]() {
-    if (cb.issued >= total_steps) return;
-    if (--cb.left == 0) {
-      cb.item += walk.slots;
-      setup_b(cb.item);
-    } else if (++cb.kt == cb.kt_end) {
-      cb.kt = cb.kt_begin;
+  auto advance_b = [&](auto plain_tag) {
+    if (!decltype(plain_tag)::value) {
+      if (cb.issued >= total_steps) return;
+      if (--cb.left == 0) {
+        cb.item += walk.slots;
+        setup_b(cb.item);
+        return;
+      }
+    } else {
+      --cb.left;
     }
+    cb.kt = (cb.kt + 1 == cb.kt_end) ? cb.kt_begin : cb.kt + 1;
   };
 
   // ---- operand fragments: two register sets; each fragment is two 16-byte LDS reads
@@ -549,8 +558,8 @@ void gemm_tiled_kernel(GemmParams p) {
   setup_b(cb.item);
 #pragma unroll
   for (int d = 0; d < DIST; ++d) {
-    issue_a(); advance_a();
-    issue_b(); advance_b();
+    issue_a(); advance_a(std::false_type{});
+    issue_b(); advance_b(std::false_type{});
   }
   wait_loads_and_barrier<(DIST - 1) * (A_GROUPS + B_GROUPS)>();
 #pragma unroll
@@ -717,44 +726,76 @@ void gemm_tiled_kernel(GemmParams p) {
   };
 
   int sa = 0, sb = 0;  // stages holding the step being computed
+  const uint8_t* cur_a = lds + a_rd_base;  // where this wave reads the step being computed ...
+  const uint8_t* cur_b = lds + b_rd_base;
+  const uint8_t* nxt_a = cur_a;            // ... and the step after it
+  const uint8_t* nxt_b = cur_b;
+  // What a phase's loads need, put together while the previous phase's last MFMAs run: between
+  // the last MFMA of one phase and the first of the next a wave, which issues its instructions in
+  // order, should find as little as possible (every scalar instruction there is time the matrix
+  // pipe waits once its 64 cycles of cover are used up).
+  struct LoadPhase {
+    uint32_t lane_off, step_off;
+    uint8_t* stage;
+  };
+  LoadPhase ph_a = {0, 0, lds}, ph_b = {0, 0, lds};  // loads of A (issued in phase [B]) / of B (issued in phase [A])
+  auto prepare_b_loads = [&]() {
+    ph_b.lane_off = lane_part(b_lane, b_lane_tail, cb.kt);
+    ph_b.step_off = (uint32_t)cb.kt * kStepK + b_src.wave_off;
+    ph_b.stage = lds + LDS_B0 + fill_b * STAGE_B;
+    next_fill_b();
+    ++cb.issued;
+  };
+  auto prepare_a_loads = [&]() {
+    ph_a.lane_off = lane_part(a_lane, a_lane_tail, ca.kt);
+    ph_a.step_off = (uint32_t)ca.kt * kStepK + a_src.wave_off;
+    ph_a.stage = lds + fill_a * STAGE_A;
+    next_fill_a();
+    ++ca.issued;
+  };
+  constexpr int B_LAST = (B_GROUPS - 1) * NMFMA / B_GROUPS;  // slots of a phase's last load
+  constexpr int A_LAST = (A_GROUPS - 1) * NMFMA / A_GROUPS;
   // One K step. READ_NEXT: fetch the first-half fragments of the following step behind the
   // second-half MFMAs (left out on a tile's last step, so that the epilogue has those
   // registers; the fragments are then read after it).
-  auto step = [&](auto first_tag, auto read_next_tag) {
+  // PLAIN: neither load cursor leaves its work item in this step.
+  // slots behind which the next phase is prepared (two, so that neither holds more scalar work than
+  // an MFMA covers)
+  constexpr int PREP_T = NMFMA / 2, PREP_T2 = NMFMA >= 8 ? NMFMA / 2 + 1 : NMFMA / 2;
+  auto step = [&](auto first_tag, auto read_next_tag, auto plain_tag) {
     constexpr bool FIRST = decltype(first_tag)::value;
     constexpr bool READ_NEXT = decltype(read_next_tag)::value;
-    const uint8_t* cur_a = lds + a_rd_base + sa * STAGE_A;
-    const uint8_t* cur_b = lds + b_rd_base + sb * STAGE_B;
-    sa = (sa + 1 == kStagesA) ? 0 : sa + 1;
-    sb = (sb + 1 == kStagesB) ? 0 : sb + 1;
-    const uint8_t* nxt_a = lds + a_rd_base + sa * STAGE_A;
-    const uint8_t* nxt_b = lds + b_rd_base + sb * STAGE_B;
 
     // [A] MFMAs on x* (first K half of this step). Behind them, one per MFMA: the LDS reads
     //     of the second half (-> y*), and behind every other one a global->LDS load of
     //     B(g+DIST) into the B stage released at the previous barrier. The fences pin this
     //     interleaving: every wave-level memory instruction hides behind an MFMA, and the
-    //     load queue never holds more than the matrix pipe can cover.
+    //     load queue never holds more than the matrix pipe can cover. Half way through, phase [B]
+    //     is prepared; behind the last loads the B cursor moves on. Behind the phase's last MFMA
+    //     there is nothing but the wait and the barrier, which its 64 cycles cover.
     __builtin_amdgcn_sched_barrier(0);
-    {
-      const uint8_t* gb = l_b + (size_t)cb.kt * kStepK;
-      const bool real = !KTAIL || cb.kt < k_full || tail_chunk_ok;
-      uint8_t* wb = lds + LDS_B0 + (cb.issued % kStagesB) * STAGE_B + wave * 1024;
-      ++cb.issued;
 #pragma unroll
-      for (int t = 0; t < NMFMA; ++t) {
-        if (BLOCKSCALE) fold_block(t, FIRST);  // the previous step's block t, before it is overwritten
-        mfma_one(xa, xb, t, BLOCKSCALE || FIRST);
+    for (int t = 0; t < NMFMA; ++t) {
+      if (BLOCKSCALE) fold_block(t, FIRST);  // the previous step's block t, before it is overwritten
+      mfma_one(xa, xb, t, BLOCKSCALE || FIRST);
+      __builtin_amdgcn_sched_barrier(0);  // the MFMA goes first: what follows is issued under its cover
 #pragma unroll
-        for (int l = 0; l < B_GROUPS; ++l)
-          if (l * NMFMA / B_GROUPS == t) load_chunk_to_lds<STREAM_B>(chunk_src(gb, b_off, l, real), wb + NW * l * 1024);
+      for (int l = 0; l < B_GROUPS; ++l)
+        if (l * NMFMA / B_GROUPS == t)
+          load_group(std::integral_constant<bool, STREAM_B>{}, b_src, ph_b.lane_off, ph_b.step_off, l, ph_b.stage);
 #pragma unroll
-        for (int u = t * RPS; u < (t + 1) * RPS; ++u)
-          if (u < NREAD) read_one(ya, yb, cur_a, cur_b, 1, u);
-        __builtin_amdgcn_sched_barrier(0);
+      for (int u = t * RPS; u < (t + 1) * RPS; ++u)
+        if (u < NREAD) read_one(ya, yb, cur_a, cur_b, 1, u);
+      if (t == B_LAST) advance_b(plain_tag);
+      if (t == PREP_T) prepare_a_loads();
+      if (t == PREP_T2) {
+        sa = (sa + 1 == kStagesA) ? 0 : sa + 1;
+        sb = (sb + 1 == kStagesB) ? 0 : sb + 1;
+        nxt_a = lds + a_rd_base + sa * STAGE_A;
+        nxt_b = lds + b_rd_base + sb * STAGE_B;
       }
+      __builtin_amdgcn_sched_barrier(0);
     }
-    advance_b();
 
     // own loads of A(g+1) and B(g+1) have landed (the younger B(g+2) .. B(g+DIST) and
     // A(g+2) .. A(g+DIST-1) may still be in flight); past the barrier everyone's have, and
@@ -765,36 +806,36 @@ void gemm_tiled_kernel(GemmParams p) {
     //     released and the LDS reads of step g+1's first half (-> x*; at the end of a tile
     //     these already belong to the next tile)
     __builtin_amdgcn_sched_barrier(0);
-    {
-      const uint8_t* ga = l_a + (size_t)ca.kt * kStepK;
-      const bool real = !KTAIL || ca.kt < k_full || tail_chunk_ok;
-      uint8_t* wa = lds + (ca.issued % kStagesA) * STAGE_A + wave * 1024;
-      ++ca.issued;
 #pragma unroll
-      for (int t = 0; t < NMFMA; ++t) {
-        mfma_one(ya, yb, t, false);
+    for (int t = 0; t < NMFMA; ++t) {
+      mfma_one(ya, yb, t, false);
+      __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-        for (int l = 0; l < A_GROUPS; ++l)
-          if (l * NMFMA / A_GROUPS == t) load_chunk_to_lds(chunk_src(ga, a_off, l, real), wa + NW * l * 1024);
+      for (int l = 0; l < A_GROUPS; ++l)
+        if (l * NMFMA / A_GROUPS == t) load_group(std::false_type{}, a_src, ph_a.lane_off, ph_a.step_off, l, ph_a.stage);
 #pragma unroll
-        for (int u = t * RPS; u < (t + 1) * RPS; ++u)
-          if (READ_NEXT && u < NREAD) read_one(xa, xb, nxt_a, nxt_b, 0, u);
-        __builtin_amdgcn_sched_barrier(0);
+      for (int u = t * RPS; u < (t + 1) * RPS; ++u)
+        if (READ_NEXT && u < NREAD) read_one(xa, xb, nxt_a, nxt_b, 0, u);
+      if (t == A_LAST) advance_a(plain_tag);
+      if (t == PREP_T) {
+        prepare_b_loads();
+        cur_a = nxt_a;
+        cur_b = nxt_b;
       }
+      __builtin_amdgcn_sched_barrier(0);
     }
-    advance_a();
     if (BLOCKSCALE) s_pend = step_scale(kt_c++);
   };
   auto read_first_half = [&]() {
 #pragma unroll
-    for (int u = 0; u < NREAD; ++u)
-      read_one(xa, xb, lds + a_rd_base + sa * STAGE_A, lds + b_rd_base + sb * STAGE_B, 0, u);
+    for (int u = 0; u < NREAD; ++u) read_one(xa, xb, cur_a, cur_b, 0, u);
   };
 
   // Item loop around the K loop. The first step of an item is its own copy of the step code
   // whose first-half MFMAs start from zero: the accumulators then have one live range per
   // item (defined there, dead after the epilogue) and need no clearing or copying between
   // items.
+  prepare_b_loads();  // of the first step's phase [A]
   for (int c_item = walk.slot; c_item < walk.chunk_len; c_item += walk.slots) {
     const int c_split = item_split(c_item);
     const int n_steps = split_end(c_split) - split_begin(c_split);
@@ -803,11 +844,15 @@ void gemm_tiled_kernel(GemmParams p) {
       kt_c = split_begin(c_split);
     }
     if (n_steps == 1) {
-      step(std::true_type{}, std::false_type{});
+      step(std::true_type{}, std::false_type{}, std::false_type{});
     } else {
-      step(std::true_type{}, std::true_type{});
-      for (int k = 2; k < n_steps; ++k) step(std::false_type{}, std::true_type{});
-      step(std::false_type{}, std::false_type{});
+      // step k loads for step k + DIST and then moves the cursors to step k + DIST + 1, which is
+      // still this item's for k < n_steps - DIST - 1
+      step(std::true_type{}, std::true_type{}, std::false_type{});
+      int k = 1;
+      for (; k < n_steps - DIST - 1; ++k) step(std::false_type{}, std::true_type{}, std::true_type{});
+      for (; k < n_steps - 1; ++k) step(std::false_type{}, std::true_type{}, std::false_type{});
+      step(std::false_type{}, std::false_type{}, std::false_type{});
     }
     if (BLOCKSCALE) {
 #pragma unroll
@@ -1097,14 +1142,16 @@ __global__ __launch_bounds__(KW * 64) void gemm_skinny_kernel(GemmParams p) {
 }
 
 // ------------------------------------------------------------------------------------
-// Persistent skinny kernel for M <= 16 and K = 16*SPW 128-byte steps (K = 2048 .. 8192): one
-// workgroup of 16 waves per CU walks a contiguous run of 16-row tiles of B. Wave w owns the K
-// steps w, w+16, ... of every tile and keeps its share of A (SPW fragments, 8 registers each)
-// in registers for the whole launch: A crosses the L2->L1 path once per CU instead of once per
-// tile, which is where the one-tile-per-workgroup kernel above loses a tenth of its time at
-// M = 16. The loads of B run one tile (SPW steps) ahead of their use; per tile the waves'
-// partial 16x16 results meet in LDS (two alternating areas, one barrier per tile) and one wave,
-// a different one for every tile, adds them in wave order and stores.
+// Persistent skinny kernel for M <= 16*MT (MT = 1, 2) and K = 16*SPW 128-byte steps (K = 2048 ..
+// 8192): one workgroup of 16 waves per CU walks a contiguous run of 16-row tiles of B. Wave w
+// owns the K steps w, w+16, ... of every tile and keeps its share of A (MT*SPW fragments, 8
+// registers each) in registers for the whole launch: A crosses the L2->L1 path once per CU
+// instead of once per tile, which is where the one-tile-per-workgroup kernel above loses a
+// tenth of its time at M = 16 and a quarter at M = 32. The loads of B run LAG steps ahead of
+// their use (a whole tile with one block of A; two steps with two, whose fragments take the
+// registers); per tile the waves' partial 16x16 results meet in LDS (two alternating areas, one
+// barrier per tile) and one wave per 16x16 result, a different one every time, adds them in
+// wave order and stores.
 // Workgroup g starts its K walk at step 2*(g/8) (workgroups g, g+8, ... share an XCD): the
 // workgroups of an XCD then ask its L2 for different lines of A at any one time, and the
 // addresses of B in flight do not all agree in their low bits (measured at N=K=8192, M=16:
@@ -1112,16 +1159,19 @@ __global__ __launch_bounds__(KW * 64) void gemm_skinny_kernel(GemmParams p) {
 // ------------------------------------------------------------------------------------
 constexpr int kPersistWaves = 16;
 
+constexpr size_t persistent_lds_bytes(int MT) { return (size_t)kPersistWaves * 2048 + (size_t)2 * kPersistWaves * MT * 1024; }
+
 // VEC: b_scale, bias and C are aligned for 16-, 8- and 8-byte accesses (else element by element).
-template <int SPW, bool VEC>
+template <int SPW, int MT, int LAG, bool VEC>
 __global__ __launch_bounds__(kPersistWaves * 64) void gemm_skinny_persistent_kernel(GemmParams p) {
   constexpr int WAVES = kPersistWaves;
   constexpr int STEPS = WAVES * SPW;
+  static_assert(LAG >= 1 && LAG <= SPW && SPW % LAG == 0, "the landing registers are a ring of LAG steps");
   extern __shared__ __attribute__((aligned(1024))) uint8_t lds[];
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   uint8_t* buf = lds + wave * 2048;             // this wave's transpose buffer (one 16 x 128 B step)
-  v4f* red = (v4f*)(lds + WAVES * 2048);        // [2][WAVES][64] partial results
+  v4f* red = (v4f*)(lds + WAVES * 2048);        // [2][MT][WAVES][64] partial results
 
   // this workgroup's run of tiles: the first `rem` workgroups take one tile more (quotient and
   // remainder of tiles by workgroups come from the host: the division would sit in front of the
@@ -1161,29 +1211,30 @@ __global__ __launch_bounds__(kPersistWaves * 64) void gemm_skinny_persistent_ker
   const int rd0 = r16 * kStepK + (((2 * g4) ^ swz128(r16)) * kChunk);
   const int rd1 = r16 * kStepK + (((2 * g4 + 1) ^ swz128(r16)) * kChunk);
 
-  v4i land[SPW][2];
+  v4i land[LAG][2];
   const size_t tile_pitch = (size_t)16 * p.ldb;
-  size_t next_tile = uniform((size_t)tile0 * tile_pitch);  // byte offset of the tile the loads are at
-  auto fetch = [&](int i) {
-    const uint8_t* sbase = p.b + (next_tile + kofs[i]);
+  size_t cur_tile = uniform((size_t)tile0 * tile_pitch);  // byte offset of the tile being multiplied
+  auto fetch = [&](int slot, size_t tile_off, int i) {
+    const uint8_t* sbase = p.b + (tile_off + kofs[i]);
 #pragma unroll
-    for (int h = 0; h < 2; ++h) land[i][h] = __builtin_nontemporal_load((const v4i*)(sbase + b_lane[h]));
+    for (int h = 0; h < 2; ++h) land[slot][h] = __builtin_nontemporal_load((const v4i*)(sbase + b_lane[h]));
   };
-  // The first tile's rows of B are asked for before anything else: they come from HBM.
+  // The first rows of B are asked for before anything else: they come from HBM.
 #pragma unroll
-  for (int i = 0; i < SPW; ++i) fetch(i);
+  for (int i = 0; i < LAG; ++i) fetch(i, cur_tile, i);
   __builtin_amdgcn_sched_barrier(0);
   // A: whole-line loads (8 lanes per row, rows past M repeat the last one), turned into the
-  // MFMA lane layout through the transpose buffer, once
-  v8i fa[SPW];
-  {
+  // MFMA lane layout through the transpose buffer, once, one 16-row block at a time
+  v8i fa[MT][SPW];
+#pragma unroll
+  for (int u = 0; u < MT; ++u) {
     v4i la[SPW][2];
 #pragma unroll
     for (int i = 0; i < SPW; ++i) {
       const uint8_t* sbase = p.a + kofs[i];
 #pragma unroll
       for (int h = 0; h < 2; ++h)
-        la[i][h] = *(const v4i*)(sbase + ((uint32_t)min(h * 8 + ld_row, p.M - 1) * (uint32_t)p.lda + ld_c * kChunk));
+        la[i][h] = *(const v4i*)(sbase + ((uint32_t)min(u * 16 + h * 8 + ld_row, p.M - 1) * (uint32_t)p.lda + ld_c * kChunk));
     }
     __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
@@ -1192,23 +1243,26 @@ __global__ __launch_bounds__(kPersistWaves * 64) void gemm_skinny_persistent_ker
       *(v4i*)(buf + wr_off[1]) = la[i][1];
       const v4i lo = *(const v4i*)(buf + rd0);
       const v4i hi = *(const v4i*)(buf + rd1);
-      fa[i] = (v8i){lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+      fa[u][i] = (v8i){lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
     }
+    __builtin_amdgcn_sched_barrier(0);
   }
-  // Wave w finishes the tiles j = w, w + 16, ... of the run: lane (m = lane % 16, quad lane / 16)
-  // owns C[m, 16*tile + 4*(lane/16) .. +3]. The column scales and bias of a wave's next tile are
-  // fetched long before they are used (here, and after each finished tile) and kept as loaded;
-  // a run without a tile for this wave reads the run's last tile instead.
-  const float fin_sa = p.a_scale[min(r16, p.M - 1)];
+  // The 16x16 results are numbered q = MT*j + u (tile j of the run, block u of A); wave w finishes
+  // the results q = w, w + 16, ...: lane (m = 16u + lane % 16, quad lane / 16) owns
+  // C[m, 16*tile + 4*(lane/16) .. +3]. The column scales and bias of a wave's next result are
+  // fetched long before they are used (here, and after each finished result) and kept as loaded;
+  // a run without a result for this wave reads the run's last tile instead.
   // Without a bias the same loads read the head of b_scale instead and the bits are masked off:
   // the loads stay unconditional and in the global address space either way.
   const uint16_t* const bias_src = p.bias ? p.bias : reinterpret_cast<const uint16_t*>(p.b_scale);
   const int bias_stride = p.bias ? 1 : 0;
   const uint16_t bias_mask = p.bias ? 0xffffu : 0u;
-  float sb_raw[4];
+  float sb_raw[4], fin_sa;
   uint16_t bias_raw[4];
-  auto load_epi = [&](int j) {
-    const int n = (tile0 + min(j, count - 1)) * 16 + 4 * g4;
+  auto load_epi = [&](int qi) {
+    const int qc = min(qi, count * MT - 1);
+    const int n = (tile0 + qc / MT) * 16 + 4 * g4;
+    fin_sa = p.a_scale[min((qc % MT) * 16 + r16, p.M - 1)];
     if (VEC) {
       const v4f s4 = *(const v4f*)(p.b_scale + n);
       const us4 b4 = *(const us4*)(bias_src + n * bias_stride);
@@ -1221,59 +1275,76 @@ __global__ __launch_bounds__(kPersistWaves * 64) void gemm_skinny_persistent_ker
   };
   load_epi(wave);
 
-  auto consume = [&](int i, v4f& acc) {
-    *(v4i*)(buf + wr_off[0]) = land[i][0];
-    *(v4i*)(buf + wr_off[1]) = land[i][1];
+  auto consume = [&](int slot, int i, v4f (&acc)[MT]) {
+    *(v4i*)(buf + wr_off[0]) = land[slot][0];
+    *(v4i*)(buf + wr_off[1]) = land[slot][1];
     const v4i lo = *(const v4i*)(buf + rd0);
     const v4i hi = *(const v4i*)(buf + rd1);
     const v8i fb = (v8i){lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
-    acc = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(fb, fa[i], acc, 0, 0, 0, 0, 0, 0);
+#pragma unroll
+    for (int u = 0; u < MT; ++u)
+      acc[u] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(fb, fa[u][i], acc[u], 0, 0, 0, 0, 0, 0);
   };
-  auto finish = [&](int j, const v4f& acc) {
-    v4f* area = red + (j & 1) * WAVES * 64;
-    area[wave * 64 + lane] = acc;
+  auto finish = [&](int j, const v4f (&acc)[MT]) {
+    v4f* area = red + (j & 1) * (MT * WAVES * 64);
+#pragma unroll
+    for (int u = 0; u < MT; ++u) area[(u * WAVES + wave) * 64 + lane] = acc[u];
     __syncthreads();
     // (the area is written again two tiles later, behind the next barrier, which the finishing
-    // wave reaches only after these reads)
-    if (wave == (j & (WAVES - 1))) {
-      v4f sum = {0.f, 0.f, 0.f, 0.f};
+    // waves reach only after these reads)
+#pragma unroll
+    for (int u = 0; u < MT; ++u) {
+      if (wave == ((j * MT + u) & (WAVES - 1))) {
+        const v4f* part = area + u * WAVES * 64 + lane;
+        v4f sum = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll 1
-      for (int w0 = 0; w0 < WAVES; w0 += 8) {  // eight partials in flight at a time: all sixteen cost 64 registers
+        for (int w0 = 0; w0 < WAVES; w0 += 8) {  // eight partials in flight at a time: all sixteen cost 64 registers
 #pragma unroll
-        for (int w = 0; w < 8; ++w) sum += area[(w0 + w) * 64 + lane];
-      }
-      if (r16 < p.M) {
-        float r[4];
-#pragma unroll
-        for (int x = 0; x < 4; ++x) r[x] = __builtin_fmaf(sum[x] * fin_sa, sb_raw[x], bf16_to_f32(bias_raw[x] & bias_mask));
-        const uint32_t lo = pack_out_x2(r[0], r[1], p.out_f16), hi = pack_out_x2(r[2], r[3], p.out_f16);
-        uint16_t* dst = p.c + (size_t)r16 * p.ldc + (tile0 + j) * 16 + 4 * g4;
-        if (VEC) {
-          *(v2u*)dst = (v2u){lo, hi};
-        } else {
-          dst[0] = (uint16_t)lo; dst[1] = (uint16_t)(lo >> 16);
-          dst[2] = (uint16_t)hi; dst[3] = (uint16_t)(hi >> 16);
+          for (int w = 0; w < 8; ++w) sum += part[(w0 + w) * 64];
         }
+        const int m = u * 16 + r16;
+        if (m < p.M) {
+          float r[4];
+#pragma unroll
+          for (int x = 0; x < 4; ++x) r[x] = __builtin_fmaf(sum[x] * fin_sa, sb_raw[x], bf16_to_f32(bias_raw[x] & bias_mask));
+          const uint32_t lo = pack_out_x2(r[0], r[1], p.out_f16), hi = pack_out_x2(r[2], r[3], p.out_f16);
+          uint16_t* dst = p.c + (size_t)m * p.ldc + (tile0 + j) * 16 + 4 * g4;
+          if (VEC) {
+            *(v2u*)dst = (v2u){lo, hi};
+          } else {
+            dst[0] = (uint16_t)lo; dst[1] = (uint16_t)(lo >> 16);
+            dst[2] = (uint16_t)hi; dst[3] = (uint16_t)(hi >> 16);
+          }
+        }
+        load_epi(j * MT + u + WAVES);
       }
-      load_epi(j + WAVES);
     }
   };
 
   int j = 0;
   for (; j + 1 < count; ++j) {
-    next_tile = uniform(next_tile + tile_pitch);
-    v4f acc = {0.f, 0.f, 0.f, 0.f};
+    const size_t next_tile = uniform(cur_tile + tile_pitch);
+    v4f acc[MT];
+#pragma unroll
+    for (int u = 0; u < MT; ++u) acc[u] = (v4f){0.f, 0.f, 0.f, 0.f};
 #pragma unroll
     for (int i = 0; i < SPW; ++i) {
-      consume(i, acc);
-      fetch(i);
+      consume(i % LAG, i, acc);
+      if (i + LAG < SPW) fetch(i % LAG, cur_tile, i + LAG);
+      else fetch(i % LAG, next_tile, i + LAG - SPW);
     }
     finish(j, acc);
+    cur_tile = next_tile;
   }
   {
-    v4f acc = {0.f, 0.f, 0.f, 0.f};
+    v4f acc[MT];
 #pragma unroll
-    for (int i = 0; i < SPW; ++i) consume(i, acc);
+    for (int u = 0; u < MT; ++u) acc[u] = (v4f){0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int i = 0; i < SPW; ++i) {
+      consume(i % LAG, i, acc);
+      if (i + LAG < SPW) fetch(i % LAG, cur_tile, i + LAG);
+    }
     finish(j, acc);
   }
 }
@@ -1550,7 +1621,8 @@ constexpr TileConfig kTileConfigs[kNumTileConfigs] = {
 inline bool persistent_skinny_fits(int64_t M, int64_t N, int64_t K);
 inline float skinny_cost_us(int64_t M, int64_t N, int64_t K) {
   // the persistent form (measured: 12.7 us at N=K=8192, 71 us at N=57344)
-  if (persistent_skinny_fits(M, N, K)) return 3.0f + (float)N * (float)K / 6.9e6f;
+  // (two blocks of A, K = 4096: 9.9 us at N=8192)
+  if (persistent_skinny_fits(M, N, K)) return 3.0f + (float)N * (float)K / (M <= 16 ? 6.9e6f : 4.9e6f);
   static const float rate[4] = {6.0e6f, 4.5e6f, 3.44e6f, 3.6e6f};
   const int blocks = (int)((M + 15) / 16);
   const int b = blocks < 1 ? 0 : blocks > 4 ? 3 : blocks - 1;
@@ -1766,15 +1838,21 @@ int scratch_of_current_device(void** out) {
   return MI355X_FP8_OK;
 }
 
-// The persistent skinny kernel takes M <= 16 with N a multiple of 16 and K of 2048 up to 8192.
+// The persistent skinny kernel takes N a multiple of 16 and K of 2048 up to 8192 with M <= 16,
+// and K = 4096 with M <= 32. (Two blocks of A in registers leave room for two steps of B in
+// flight per wave. At K = 4096 that is a whole tile ahead and the form wins: M=32, N=8192 9.9 us
+// against 11.4 us for the one-tile kernel. At K = 8192 it is half a tile and loses, 20.6 against
+// 17.9 us; four steps in flight do not fit the 128 registers of a 16-wave workgroup.)
 inline bool persistent_skinny_fits(int64_t M, int64_t N, int64_t K) {
-  return M <= 16 && N % 16 == 0 && K % (kPersistWaves * kStepK) == 0 && K / (kPersistWaves * kStepK) <= 4;
+  if (N % 16 != 0 || K % (kPersistWaves * kStepK) != 0) return false;
+  const int64_t spw = K / (kPersistWaves * kStepK);
+  return (M <= 16 && spw <= 4) || (M <= 32 && spw == 2);
 }
 
-template <int SPW, bool VEC>
+template <int SPW, int MT, int LAG, bool VEC>
 int launch_skinny_persistent(const GemmParams& p, hipStream_t stream) {
-  constexpr size_t lds_bytes = (size_t)kPersistWaves * 2048 + 2 * kPersistWaves * 1024;
-  auto kern = gemm_skinny_persistent_kernel<SPW, VEC>;
+  constexpr size_t lds_bytes = persistent_lds_bytes(MT);
+  auto kern = gemm_skinny_persistent_kernel<SPW, MT, LAG, VEC>;
   static bool attr_done[kMaxDevices] = {};
   if (const int st = raise_lds_limit((const void*)kern, lds_bytes, attr_done)) return st;
   const long ntiles = p.N / 16;
@@ -1790,11 +1868,13 @@ int launch_skinny_persistent(const GemmParams& p, hipStream_t stream) {
 
 template <bool VEC>
 int launch_skinny_persistent_steps(const GemmParams& p, hipStream_t s) {
-  switch (p.K / (kPersistWaves * kStepK)) {
-    case 1: return launch_skinny_persistent<1, VEC>(p, s);
-    case 2: return launch_skinny_persistent<2, VEC>(p, s);
-    case 3: return launch_skinny_persistent<3, VEC>(p, s);
-    default: return launch_skinny_persistent<4, VEC>(p, s);
+  const int spw = p.K / (kPersistWaves * kStepK);
+  if (p.M > 16) return launch_skinny_persistent<2, 2, 2, VEC>(p, s);
+  switch (spw) {
+    case 1: return launch_skinny_persistent<1, 1, 1, VEC>(p, s);
+    case 2: return launch_skinny_persistent<2, 1, 2, VEC>(p, s);
+    case 3: return launch_skinny_persistent<3, 1, 3, VEC>(p, s);
+    default: return launch_skinny_persistent<4, 1, 4, VEC>(p, s);
   }
 }
 
@@ -1852,7 +1932,8 @@ int mi355x_fp8_rowwise_gemm_ex(const void* a, const void* b, const float* a_scal
   if ((reinterpret_cast<uintptr_t>(a_scale) & 3) || (reinterpret_cast<uintptr_t>(b_scale) & 3) ||
       (reinterpret_cast<uintptr_t>(c) & 1) || (reinterpret_cast<uintptr_t>(bias) & 1))
     return fail(MI355X_FP8_EINVAL, "misaligned scale, bias or output pointer");
-  if (lda * 256 > (int64_t)UINT32_MAX || ldb * 256 > (int64_t)UINT32_MAX)
+  // (a tile's rows are addressed with 32-bit offsets that must stay below 2^31)
+  if (lda * 256 > (int64_t)INT32_MAX || ldb * 256 > (int64_t)INT32_MAX)
     return fail(MI355X_FP8_ENOTSUP, "leading dimension too large");
   if (variant < 0 || (variant >> 24) || ((variant >> 8) & 0xff) > kNumTileConfigs)
     return fail(MI355X_FP8_EINVAL, "unknown variant 0x%x", variant);
@@ -1969,7 +2050,8 @@ int mi355x_fp8_rowwise_grouped_gemm(const void* a, const void* b, const float* a
   if ((reinterpret_cast<uintptr_t>(a_scale) & 3) || (reinterpret_cast<uintptr_t>(b_scale) & 3) ||
       (reinterpret_cast<uintptr_t>(c) & 1) || (reinterpret_cast<uintptr_t>(m_sizes) & 3))
     return fail(MI355X_FP8_EINVAL, "misaligned scale, size or output pointer");
-  if (lda * 256 > (int64_t)UINT32_MAX || ldb * 256 > (int64_t)UINT32_MAX)
+  // (a tile's rows are addressed with 32-bit offsets that must stay below 2^31)
+  if (lda * 256 > (int64_t)INT32_MAX || ldb * 256 > (int64_t)INT32_MAX)
     return fail(MI355X_FP8_ENOTSUP, "leading dimension too large");
   if (tile_config < -1 || tile_config >= kNumGroupedTileConfigs)
     return fail(MI355X_FP8_EINVAL, "unknown tile configuration %d", tile_config);
@@ -2014,7 +2096,8 @@ int mi355x_fp8_blockwise_gemm(const void* a, const void* b, const float* a_scale
   if ((reinterpret_cast<uintptr_t>(a_scale) & 3) || (reinterpret_cast<uintptr_t>(b_scale) & 3) ||
       (reinterpret_cast<uintptr_t>(c) & 1))
     return fail(MI355X_FP8_EINVAL, "misaligned scale or output pointer");
-  if (lda * 256 > (int64_t)UINT32_MAX || ldb * 256 > (int64_t)UINT32_MAX)
+  // (a tile's rows are addressed with 32-bit offsets that must stay below 2^31)
+  if (lda * 256 > (int64_t)INT32_MAX || ldb * 256 > (int64_t)INT32_MAX)
     return fail(MI355X_FP8_ENOTSUP, "leading dimension too large");
   GemmParams p;
   p.a = (const uint8_t*)a; p.b = (const uint8_t*)b;
