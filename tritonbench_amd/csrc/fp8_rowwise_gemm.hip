@@ -176,6 +176,15 @@ __device__ __forceinline__ void load_chunk_to_lds(__amdgpu_buffer_rsrc_t rsrc, u
 #endif
 }
 
+// One wave-wide streaming store of 16 bytes per lane through a buffer descriptor (address = base +
+// lane_off + wave_off): the output is written once and read by a later kernel at best.
+__device__ __forceinline__ void store_chunk_streaming(v4i data, __amdgpu_buffer_rsrc_t rsrc, uint32_t lane_off,
+                                                      uint32_t wave_off) {
+#if defined(__HIP_DEVICE_COMPILE__)
+  __builtin_amdgcn_raw_buffer_store_b128(data, rsrc, (int)lane_off, (int)wave_off, 2);
+#endif
+}
+
 // Waits until at most VM of this wave's global loads and none of its LDS operations are
 // outstanding, then joins the workgroup barrier. Written with the s_waitcnt builtin (not
 // inline asm) so the compiler's own wait-count bookkeeping knows the LDS queue is empty
@@ -567,33 +576,42 @@ void gemm_tiled_kernel(GemmParams p) {
 
   // ---- epilogue. The MFMA leaves lane (l32, half) with row l32 of every 32x32 block and the
   // columns 8*q + 4*half + e (register 4*q + e): storing from there would touch 32 rows per
-  // instruction. Instead each 32-row block of the wave's tile is turned through LDS, PASS_J
-  // 32-column blocks at a time, as fp32 already multiplied by a_scale[m]; read back, a lane
-  // holds 8 consecutive columns of one row, multiplies by b_scale (adds the bias), rounds to
-  // bf16 once and stores 16 bytes, so a wave-wide store covers whole rows of the pass.
-  // A lane's 8 columns are the same for every row, which keeps its b_scale / bias working
-  // set at 8 values per pass column group.
+  // instruction. Instead a lane finishes its own elements first - a_scale[m], b_scale[n], bias[n]
+  // in fp32, one rounding to the 16-bit output type, two results per register - and each 32-row
+  // block of the wave's tile is then turned through LDS, PASS_J 32-column blocks at a time, as
+  // 16-bit values: read back, a lane holds 8 consecutive columns of one row and stores its 16
+  // bytes, so a wave-wide store covers whole rows of the pass.
   //
   // The turn-table is the wave's own share (the 1 KB groups it fills itself) of the B stage
   // that held this tile's last step: every wave finished reading that stage before the
-  // step's barrier, and only this wave will load into these groups again. A pass row is CPR
-  // 16-byte chunks; chunk c of row r sits at chunk position c ^ key(r).
-  constexpr int PASS_J = B_GROUPS / 4;          // 32-column blocks per pass (4 KB of fp32 each)
+  // step's barrier, and only this wave will load into these groups again. A pass fills half of
+  // it, so the passes alternate between two halves: while one pass is read back and stored, the
+  // next is converted and written (LDS runs a wave's operations in order, so neither half needs
+  // a wait before it is written again). A pass row is CPR 16-byte chunks; chunk c of row r sits
+  // at chunk position c ^ key(r): the 16-byte reads of 8 lanes spread over all banks, the 8-byte
+  // writes of 16 consecutive rows meet in pairs (a two-way conflict on 64 of the epilogue's
+  // instructions, which are bound by their arithmetic; undoing it costs the readers register moves).
+  constexpr int PASS_J = B_GROUPS / 4;          // 32-column blocks per pass (2 KB of 16-bit values each)
   constexpr int NJP = NT / PASS_J;              // passes per 32-row block
-  constexpr int CPR = PASS_J * 8;               // 16-byte chunks per pass row
+  constexpr int CPR = PASS_J * 4;               // 16-byte chunks per pass row
   constexpr int ROW_BYTES = CPR * 16;
   constexpr int ROWS_PER_GROUP = 1024 / ROW_BYTES;
-  constexpr int LPR = CPR / 2;                  // lanes per row when reading back (2 chunks each)
+  constexpr int GROUPS_PER_PASS = 32 / ROWS_PER_GROUP;  // = B_GROUPS / 2
+  constexpr int LPR = CPR;                      // lanes per row when reading back (one chunk each)
   constexpr int ROWS_PER_READ = 64 / LPR;
-  static_assert(B_GROUPS % 4 == 0 && NT % PASS_J == 0 && (CPR == 8 || CPR == 16), "turn-table geometry");
-  auto epilogue = [&](const TileLoc& loc, auto aligned_tag, uint8_t* free_b_stage) {
+  constexpr int ITERS = 32 / ROWS_PER_READ;
+  static_assert(B_GROUPS % 4 == 0 && NT % PASS_J == 0 && (CPR == 4 || CPR == 8) && 2 * GROUPS_PER_PASS == B_GROUPS,
+                "turn-table geometry");
+  auto epilogue = [&](const TileLoc& loc, auto aligned_tag, auto f16_tag, uint8_t* free_b_stage) {
     const int m0 = loc.m0, n0 = loc.n0;
     const float* const b_scale = p.b_scale + (GROUPED ? (size_t)loc.group * p.N : 0);
     constexpr bool ALIGNED = decltype(aligned_tag)::value;  // whole tile inside C, rows 16-byte aligned
-    auto row_addr = [&](int r) -> uint8_t* {
-      return free_b_stage + (wave + NW * (r / ROWS_PER_GROUP)) * 1024 + (r % ROWS_PER_GROUP) * ROW_BYTES;
+    constexpr bool OUT_F16 = decltype(f16_tag)::value;      // IEEE binary16 instead of bf16
+    // row r of the pass kept in half h of the table
+    auto row_addr = [&](int h, int r) -> uint8_t* {
+      return free_b_stage + (wave + NW * (h * GROUPS_PER_PASS + r / ROWS_PER_GROUP)) * 1024 + (r % ROWS_PER_GROUP) * ROW_BYTES;
     };
-    auto key = [](int r) { return (r * CPR / 16) % CPR; };
+    auto key = [](int r) { return (r * ROW_BYTES / 128) % CPR; };
     // The lane-dependent addresses below are the same for every tile; derived from an opaque
     // copy of the lane id they are recomputed here (a few integer operations) instead of
     // being hoisted out of the tile loop, where they would occupy registers through the K loop.
@@ -601,93 +619,107 @@ void gemm_tiled_kernel(GemmParams p) {
     int lane_e = (int)__builtin_amdgcn_mbcnt_hi(~0u, __builtin_amdgcn_mbcnt_lo(~0u, 0u));
     asm volatile("" : "+v"(lane_e));
     const int l32 = lane_e & 31, half = lane_e >> 5;
-    uint8_t* const wr_row = row_addr(l32);
     const int wr_key = key(l32);
-    const int rd_row = lane_e / LPR, rd_col = (lane_e % LPR) * 8;  // column of the pass row this lane stores
+    const int wr_half = half * 8;  // where this lane's 8 bytes sit inside a chunk
+    const int rd_row = lane_e / LPR, rd_chunk = lane_e % LPR;  // 8 columns of the pass row this lane stores
+    const int rd_col = rd_chunk * 8;
 
-    float sam[MT], sbv[NJP][8], bv[NJP][8];
+    // scales and bias of the lane's own elements: row l32 of every 32-row block, columns
+    // 32*j + 8*q + 4*half + e
+    // (the bias stays as loaded, two bf16 per register, and is widened where it is used)
+    float sam[MT], sbv[NT][4][4];
+    us4 bv[HAS_BIAS ? NT : 1][4];
 #pragma unroll
     for (int i = 0; i < MT; ++i)
       sam[i] = BLOCKSCALE ? 1.0f : p.a_scale[min(m0 + wm * WTM + i * 32 + l32, loc.m_end - 1)];
 #pragma unroll
-    for (int jp = 0; jp < NJP; ++jp) {
-      const int n = n0 + wn * WTN + jp * PASS_J * 32 + rd_col;
-      if (BLOCKSCALE) {  // the factors were applied step by step
+    for (int j = 0; j < NT; ++j) {
 #pragma unroll
-        for (int e = 0; e < 8; ++e) sbv[jp][e] = 1.0f;
-      } else if (ALIGNED) {
-        const v4f s0 = *(const v4f*)(b_scale + n), s1 = *(const v4f*)(b_scale + n + 4);
+      for (int q = 0; q < 4; ++q) {
+        const int n = n0 + wn * WTN + j * 32 + 8 * q + 4 * half;
+        if (BLOCKSCALE) {  // the factors were applied step by step
 #pragma unroll
-        for (int e = 0; e < 4; ++e) sbv[jp][e] = s0[e], sbv[jp][4 + e] = s1[e];
-        if (HAS_BIAS) {
-          const us4 b0 = *(const us4*)(p.bias + n), b1 = *(const us4*)(p.bias + n + 4);
+          for (int e = 0; e < 4; ++e) sbv[j][q][e] = 1.0f;
+        } else if (ALIGNED) {
+          const v4f s4 = *(const v4f*)(b_scale + n);
 #pragma unroll
-          for (int e = 0; e < 4; ++e) bv[jp][e] = bf16_to_f32(b0[e]), bv[jp][4 + e] = bf16_to_f32(b1[e]);
-        }
-      } else {
+          for (int e = 0; e < 4; ++e) sbv[j][q][e] = s4[e];
+          if (HAS_BIAS) bv[HAS_BIAS ? j : 0][q] = *(const us4*)(p.bias + n);
+        } else {
 #pragma unroll
-        for (int e = 0; e < 8; ++e) {
-          sbv[jp][e] = b_scale[min(n + e, p.N - 1)];
-          if (HAS_BIAS) bv[jp][e] = bf16_to_f32(p.bias[min(n + e, p.N - 1)]);
+          for (int e = 0; e < 4; ++e) {
+            sbv[j][q][e] = b_scale[min(n + e, p.N - 1)];
+            if (HAS_BIAS) bv[HAS_BIAS ? j : 0][q][e] = p.bias[min(n + e, p.N - 1)];
+          }
         }
       }
     }
+    // pass pp = (32-row block i, column blocks jp*PASS_J ..): finished 16-bit values into half pp & 1.
+    // One 32x32 block at a time in three sweeps over its 16 values (row scale, column scale and
+    // bias, rounding): neighbouring instructions then do not wait for each other's results.
+    auto convert_and_write = [&](int pp) {
+      const int i = pp / NJP, jp = pp % NJP;
+      uint8_t* const wr_row = row_addr(pp & 1, l32);
 #pragma unroll
-    for (int i = 0; i < MT; ++i) {
+      for (int jj = 0; jj < PASS_J; ++jj) {
+        const int j = jp * PASS_J + jj;
+        float t[16], x[16];
+        uint32_t packed[8];
 #pragma unroll
-      for (int jp = 0; jp < NJP; ++jp) {
+        for (int v = 0; v < 16; ++v) t[v] = acc[i][j][v] * sam[i];
         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-        for (int jj = 0; jj < PASS_J; ++jj) {
-          const int j = jp * PASS_J + jj;
-#pragma unroll
-          for (int q = 0; q < 4; ++q) {
-            v4f t;
-#pragma unroll
-            for (int e = 0; e < 4; ++e) t[e] = acc[i][j][4 * q + e] * sam[i];
-            *(v4f*)(wr_row + (((jj * 8 + 2 * q + half) ^ wr_key) * 16)) = t;
-          }
-          __builtin_amdgcn_sched_barrier(0);  // keeps the live set small: one block at a time
-        }
-        const int n = n0 + wn * WTN + jp * PASS_J * 32 + rd_col;
-        constexpr int ITERS = 32 / ROWS_PER_READ;
-        v4f lo4[ITERS], hi4[ITERS];
-#pragma unroll
-        for (int it = 0; it < ITERS; ++it) {
-          const int r = it * ROWS_PER_READ + rd_row;
-          const uint8_t* src = row_addr(r);
-          const int c0 = (rd_col / 4) ^ key(r);  // the lane's two chunks differ in bit 0 only
-          lo4[it] = *(const v4f*)(src + c0 * 16);
-          hi4[it] = *(const v4f*)(src + (c0 ^ 1) * 16);
-        }
+        for (int v = 0; v < 16; ++v)
+          x[v] = HAS_BIAS ? __builtin_fmaf(t[v], sbv[j][v / 4][v % 4], bf16_to_f32(bv[HAS_BIAS ? j : 0][v / 4][v % 4]))
+                          : t[v] * sbv[j][v / 4][v % 4];
         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-        for (int it = 0; it < ITERS; ++it) {
-          const int r = it * ROWS_PER_READ + rd_row;
-          float x[8];
+        for (int v = 0; v < 8; ++v) packed[v] = pack_out_x2(x[2 * v], x[2 * v + 1], OUT_F16);
+        __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-          for (int e = 0; e < 4; ++e) x[e] = lo4[it][e], x[4 + e] = hi4[it][e];
+        for (int q = 0; q < 4; ++q)
+          *(v2u*)(wr_row + (((jj * 4 + q) ^ wr_key) * 16) + wr_half) = (v2u){packed[2 * q], packed[2 * q + 1]};
+      }
+    };
+    // The wave's part of the tile as a buffer: origin at its first element, offsets below 2^31 by
+    // the host's check of ldc (interior tiles only: nothing here relies on the range check).
+    const uint32_t c_row_bytes = (uint32_t)p.ldc * 2u;
+    const __amdgpu_buffer_rsrc_t c_rsrc = __builtin_amdgcn_make_buffer_rsrc(
+        p.c + ((size_t)(m0 + wm * WTM) * p.ldc + n0 + wn * WTN), 0, 0x7fffffff, 0x00020000);
+    const uint32_t c_lane = (uint32_t)rd_row * c_row_bytes + (uint32_t)rd_col * 2u;
+    constexpr int NP = MT * NJP;
+    __builtin_amdgcn_sched_barrier(0);
+    convert_and_write(0);
 #pragma unroll
-          for (int e = 0; e < 8; ++e)
-            x[e] = HAS_BIAS ? __builtin_fmaf(x[e], sbv[jp][e], bv[jp][e]) : x[e] * sbv[jp][e];
-          v4i out;
-          if (p.out_f16) {
-            out = (v4i){(int)pack_f16x2(x[0], x[1]), (int)pack_f16x2(x[2], x[3]),
-                        (int)pack_f16x2(x[4], x[5]), (int)pack_f16x2(x[6], x[7])};
-          } else {
-            out = (v4i){(int)pack_bf16x2(x[0], x[1]), (int)pack_bf16x2(x[2], x[3]),
-                        (int)pack_bf16x2(x[4], x[5]), (int)pack_bf16x2(x[6], x[7])};
-          }
+    for (int pp = 0; pp < NP; ++pp) {
+      const int i = pp / NJP, jp = pp % NJP;
+      __builtin_amdgcn_sched_barrier(0);
+      v4i rows16[ITERS];
+#pragma unroll
+      for (int it = 0; it < ITERS; ++it) {
+        const int r = it * ROWS_PER_READ + rd_row;
+        rows16[it] = *(const v4i*)(row_addr(pp & 1, r) + ((rd_chunk ^ key(r)) * 16));
+      }
+      __builtin_amdgcn_sched_barrier(0);
+      if (pp + 1 < NP) convert_and_write(pp + 1);  // under the latency of the reads above
+      __builtin_amdgcn_sched_barrier(0);
+      const int n = n0 + wn * WTN + jp * PASS_J * 32 + rd_col;
+#pragma unroll
+      for (int it = 0; it < ITERS; ++it) {
+        const int r = it * ROWS_PER_READ + rd_row;
+        const v4i out = rows16[it];
+        if (ALIGNED) {
+          // lane part (rd_row, rd_col) + scalar part (block row, read round, pass column)
+          store_chunk_streaming(out, c_rsrc, c_lane,
+                                (uint32_t)(i * 32 + it * ROWS_PER_READ) * c_row_bytes + (uint32_t)(jp * PASS_J * 32 * 2));
+        } else {
           const int m = m0 + wm * WTM + i * 32 + r;
           uint16_t* dst = p.c + (size_t)m * p.ldc + n;
-          if (ALIGNED) {
-            __builtin_nontemporal_store(out, (v4i*)dst);  // written once, read by a later kernel at best
-          } else if (m < loc.m_end) {
+          if (m < loc.m_end) {
 #pragma unroll
             for (int e = 0; e < 8; ++e)
               if (n + e < p.N) dst[e] = (uint16_t)((unsigned)out[e / 2] >> (16 * (e & 1)));
           }
-          __builtin_amdgcn_sched_barrier(0);
         }
       }
     }
@@ -871,8 +903,14 @@ void gemm_tiled_kernel(GemmParams p) {
         const uintptr_t bits = reinterpret_cast<uintptr_t>(p.c) | (uintptr_t)(p.ldc * 2) |
                                reinterpret_cast<uintptr_t>(p.b_scale) | (reinterpret_cast<uintptr_t>(p.bias) << 1) |
                                (GROUPED ? (uintptr_t)(p.N * 4) : 0);
-        if (interior && (bits & 15) == 0) epilogue(loc, std::true_type{}, free_b);
-        else epilogue(loc, std::false_type{}, free_b);
+        // (the output type is a compile-time property of the epilogue code: one uniform branch per tile)
+        if (interior && (bits & 15) == 0) {
+          if (p.out_f16) epilogue(loc, std::true_type{}, std::true_type{}, free_b);
+          else epilogue(loc, std::true_type{}, std::false_type{}, free_b);
+        } else {
+          if (p.out_f16) epilogue(loc, std::false_type{}, std::true_type{}, free_b);
+          else epilogue(loc, std::false_type{}, std::false_type{}, free_b);
+        }
       }
     }
     read_first_half();  // of the next item's first step (landed before this item's last barrier)
@@ -1932,8 +1970,8 @@ int mi355x_fp8_rowwise_gemm_ex(const void* a, const void* b, const float* a_scal
   if ((reinterpret_cast<uintptr_t>(a_scale) & 3) || (reinterpret_cast<uintptr_t>(b_scale) & 3) ||
       (reinterpret_cast<uintptr_t>(c) & 1) || (reinterpret_cast<uintptr_t>(bias) & 1))
     return fail(MI355X_FP8_EINVAL, "misaligned scale, bias or output pointer");
-  // (a tile's rows are addressed with 32-bit offsets that must stay below 2^31)
-  if (lda * 256 > (int64_t)INT32_MAX || ldb * 256 > (int64_t)INT32_MAX)
+  // (a tile's rows are addressed with 32-bit byte offsets that must stay below 2^31)
+  if (lda * 256 > (int64_t)INT32_MAX || ldb * 256 > (int64_t)INT32_MAX || ldc * 512 > (int64_t)INT32_MAX)
     return fail(MI355X_FP8_ENOTSUP, "leading dimension too large");
   if (variant < 0 || (variant >> 24) || ((variant >> 8) & 0xff) > kNumTileConfigs)
     return fail(MI355X_FP8_EINVAL, "unknown variant 0x%x", variant);
@@ -2050,8 +2088,8 @@ int mi355x_fp8_rowwise_grouped_gemm(const void* a, const void* b, const float* a
   if ((reinterpret_cast<uintptr_t>(a_scale) & 3) || (reinterpret_cast<uintptr_t>(b_scale) & 3) ||
       (reinterpret_cast<uintptr_t>(c) & 1) || (reinterpret_cast<uintptr_t>(m_sizes) & 3))
     return fail(MI355X_FP8_EINVAL, "misaligned scale, size or output pointer");
-  // (a tile's rows are addressed with 32-bit offsets that must stay below 2^31)
-  if (lda * 256 > (int64_t)INT32_MAX || ldb * 256 > (int64_t)INT32_MAX)
+  // (a tile's rows are addressed with 32-bit byte offsets that must stay below 2^31)
+  if (lda * 256 > (int64_t)INT32_MAX || ldb * 256 > (int64_t)INT32_MAX || ldc * 512 > (int64_t)INT32_MAX)
     return fail(MI355X_FP8_ENOTSUP, "leading dimension too large");
   if (tile_config < -1 || tile_config >= kNumGroupedTileConfigs)
     return fail(MI355X_FP8_EINVAL, "unknown tile configuration %d", tile_config);
@@ -2096,8 +2134,8 @@ int mi355x_fp8_blockwise_gemm(const void* a, const void* b, const float* a_scale
   if ((reinterpret_cast<uintptr_t>(a_scale) & 3) || (reinterpret_cast<uintptr_t>(b_scale) & 3) ||
       (reinterpret_cast<uintptr_t>(c) & 1))
     return fail(MI355X_FP8_EINVAL, "misaligned scale or output pointer");
-  // (a tile's rows are addressed with 32-bit offsets that must stay below 2^31)
-  if (lda * 256 > (int64_t)INT32_MAX || ldb * 256 > (int64_t)INT32_MAX)
+  // (a tile's rows are addressed with 32-bit byte offsets that must stay below 2^31)
+  if (lda * 256 > (int64_t)INT32_MAX || ldb * 256 > (int64_t)INT32_MAX || ldc * 512 > (int64_t)INT32_MAX)
     return fail(MI355X_FP8_ENOTSUP, "leading dimension too large");
   GemmParams p;
   p.a = (const uint8_t*)a; p.b = (const uint8_t*)b;
