@@ -176,6 +176,30 @@ __device__ __forceinline__ void load_chunk_to_lds(__amdgpu_buffer_rsrc_t rsrc, u
 #endif
 }
 
+// Range-checked register loads through a buffer descriptor: 4 floats / 4 bf16 / one bf16 per lane;
+// elements past the descriptor's extent read as zero bits.
+__device__ __forceinline__ v4f load_f32x4_checked(__amdgpu_buffer_rsrc_t rsrc, uint32_t lane_off) {
+#if defined(__HIP_DEVICE_COMPILE__)
+  return __builtin_bit_cast(v4f, __builtin_amdgcn_raw_buffer_load_b128(rsrc, (int)lane_off, 0, 0));
+#else
+  return (v4f){0.f, 0.f, 0.f, 0.f};
+#endif
+}
+__device__ __forceinline__ us4 load_u16x4_checked(__amdgpu_buffer_rsrc_t rsrc, uint32_t lane_off) {
+#if defined(__HIP_DEVICE_COMPILE__)
+  return __builtin_bit_cast(us4, __builtin_amdgcn_raw_buffer_load_b64(rsrc, (int)lane_off, 0, 0));
+#else
+  return (us4){0, 0, 0, 0};
+#endif
+}
+__device__ __forceinline__ uint16_t load_u16_checked(__amdgpu_buffer_rsrc_t rsrc, uint32_t lane_off) {
+#if defined(__HIP_DEVICE_COMPILE__)
+  return __builtin_amdgcn_raw_buffer_load_b16(rsrc, (int)lane_off, 0, 0);
+#else
+  return 0;
+#endif
+}
+
 // One wave-wide streaming store of 16 bytes per lane through a buffer descriptor (address = base +
 // lane_off + wave_off): the output is written once and read by a later kernel at best.
 __device__ __forceinline__ void store_chunk_streaming(v4i data, __amdgpu_buffer_rsrc_t rsrc, uint32_t lane_off,
@@ -602,10 +626,12 @@ void gemm_tiled_kernel(GemmParams p) {
   constexpr int ITERS = 32 / ROWS_PER_READ;
   static_assert(B_GROUPS % 4 == 0 && NT % PASS_J == 0 && (CPR == 4 || CPR == 8) && 2 * GROUPS_PER_PASS == B_GROUPS,
                 "turn-table geometry");
-  auto epilogue = [&](const TileLoc& loc, auto aligned_tag, auto f16_tag, uint8_t* free_b_stage) {
+  auto epilogue = [&](const TileLoc& loc, auto vector_tag, auto f16_tag, uint8_t* free_b_stage) {
     const int m0 = loc.m0, n0 = loc.n0;
-    const float* const b_scale = p.b_scale + (GROUPED ? (size_t)loc.group * p.N : 0);
-    constexpr bool ALIGNED = decltype(aligned_tag)::value;  // whole tile inside C, rows 16-byte aligned
+    // VECTOR: C takes 16-byte stores (base and row pitch aligned, N a multiple of 8, so no lane's 8
+    // columns straddle the edge). Edge tiles take it too: rows past the edge fall outside the output
+    // descriptor's extent and lanes past column N are sent there. Anything else stores element by element.
+    constexpr bool VECTOR = decltype(vector_tag)::value;
     constexpr bool OUT_F16 = decltype(f16_tag)::value;      // IEEE binary16 instead of bf16
     // row r of the pass kept in half h of the table
     auto row_addr = [&](int h, int r) -> uint8_t* {
@@ -625,34 +651,53 @@ void gemm_tiled_kernel(GemmParams p) {
     const int rd_col = rd_chunk * 8;
 
     // scales and bias of the lane's own elements: row l32 of every 32-row block, columns
-    // 32*j + 8*q + 4*half + e
+    // 32*j + 8*q + 4*half + e, fetched through descriptors that end at column N (whatever lies
+    // past it reads as zero and belongs to columns that are never stored), four at a time
+    // whatever the alignment; only a bias that starts on an odd element is fetched one by one.
     // (the bias stays as loaded, two bf16 per register, and is widened where it is used)
     float sam[MT], sbv[NT][4][4];
     us4 bv[HAS_BIAS ? NT : 1][4];
 #pragma unroll
     for (int i = 0; i < MT; ++i)
       sam[i] = BLOCKSCALE ? 1.0f : p.a_scale[min(m0 + wm * WTM + i * 32 + l32, loc.m_end - 1)];
+    if (!BLOCKSCALE) {
+      const int n_wave = n0 + wn * WTN;               // first column of the wave's tile
+      const int n_left = max(p.N - n_wave, 0);        // columns from there to the edge
+      const __amdgpu_buffer_rsrc_t s_rsrc = __builtin_amdgcn_make_buffer_rsrc(
+          const_cast<float*>(p.b_scale) + ((GROUPED ? (size_t)loc.group * p.N : 0) + n_wave), 0, n_left * 4, 0x00020000);
+      const __amdgpu_buffer_rsrc_t bias_rsrc = __builtin_amdgcn_make_buffer_rsrc(
+          const_cast<uint16_t*>(HAS_BIAS ? p.bias + n_wave : nullptr), 0, HAS_BIAS ? n_left * 2 : 0, 0x00020000);
+      // (the check works on whole 4-byte words: with an odd N the last word of the bias is half inside.
+      // Fetched four at a time from a 4-byte aligned base that word is read whole: it cannot cross a
+      // page, and its upper half belongs to a column that is never stored.)
+      const __amdgpu_buffer_rsrc_t bias4_rsrc = __builtin_amdgcn_make_buffer_rsrc(
+          const_cast<uint16_t*>(HAS_BIAS ? p.bias + n_wave : nullptr), 0, HAS_BIAS ? ((n_left + 1) & ~1) * 2 : 0, 0x00020000);
+      const bool bias_by_four = (reinterpret_cast<uintptr_t>(p.bias) & 3) == 0;  // (n_wave is a multiple of 32)
 #pragma unroll
-    for (int j = 0; j < NT; ++j) {
+      for (int j = 0; j < NT; ++j) {
 #pragma unroll
-      for (int q = 0; q < 4; ++q) {
-        const int n = n0 + wn * WTN + j * 32 + 8 * q + 4 * half;
-        if (BLOCKSCALE) {  // the factors were applied step by step
-#pragma unroll
-          for (int e = 0; e < 4; ++e) sbv[j][q][e] = 1.0f;
-        } else if (ALIGNED) {
-          const v4f s4 = *(const v4f*)(b_scale + n);
+        for (int q = 0; q < 4; ++q) {
+          const uint32_t col = (uint32_t)(j * 32 + 8 * q + 4 * half);
+          const v4f s4 = load_f32x4_checked(s_rsrc, col * 4);
 #pragma unroll
           for (int e = 0; e < 4; ++e) sbv[j][q][e] = s4[e];
-          if (HAS_BIAS) bv[HAS_BIAS ? j : 0][q] = *(const us4*)(p.bias + n);
-        } else {
+          if (HAS_BIAS) {
+            if (bias_by_four) {
+              bv[HAS_BIAS ? j : 0][q] = load_u16x4_checked(bias4_rsrc, col * 2);
+            } else {
 #pragma unroll
-          for (int e = 0; e < 4; ++e) {
-            sbv[j][q][e] = b_scale[min(n + e, p.N - 1)];
-            if (HAS_BIAS) bv[HAS_BIAS ? j : 0][q][e] = p.bias[min(n + e, p.N - 1)];
+              for (int e = 0; e < 4; ++e) bv[HAS_BIAS ? j : 0][q][e] = load_u16_checked(bias_rsrc, (col + e) * 2);
+            }
           }
         }
       }
+    } else {  // the factors were applied step by step
+#pragma unroll
+      for (int j = 0; j < NT; ++j)
+#pragma unroll
+        for (int q = 0; q < 4; ++q)
+#pragma unroll
+          for (int e = 0; e < 4; ++e) sbv[j][q][e] = 1.0f;
     }
     // pass pp = (32-row block i, column blocks jp*PASS_J ..): finished 16-bit values into half pp & 1.
     // One 32x32 block at a time in three sweeps over its 16 values (row scale, column scale and
@@ -681,11 +726,12 @@ void gemm_tiled_kernel(GemmParams p) {
           *(v2u*)(wr_row + (((jj * 4 + q) ^ wr_key) * 16) + wr_half) = (v2u){packed[2 * q], packed[2 * q + 1]};
       }
     };
-    // The wave's part of the tile as a buffer: origin at its first element, offsets below 2^31 by
-    // the host's check of ldc (interior tiles only: nothing here relies on the range check).
+    // The wave's part of the tile as a buffer: origin at its first element, extent = its valid rows
+    // (none for a wave that lies past the edge); offsets stay below 2^31 by the host's check of ldc.
     const uint32_t c_row_bytes = (uint32_t)p.ldc * 2u;
+    const int c_rows = min(max(loc.m_end - (m0 + wm * WTM), 0), WTM);
     const __amdgpu_buffer_rsrc_t c_rsrc = __builtin_amdgcn_make_buffer_rsrc(
-        p.c + ((size_t)(m0 + wm * WTM) * p.ldc + n0 + wn * WTN), 0, 0x7fffffff, 0x00020000);
+        p.c + ((size_t)(m0 + wm * WTM) * p.ldc + n0 + wn * WTN), 0, (int)((uint32_t)c_rows * c_row_bytes), 0x00020000);
     const uint32_t c_lane = (uint32_t)rd_row * c_row_bytes + (uint32_t)rd_col * 2u;
     constexpr int NP = MT * NJP;
     __builtin_amdgcn_sched_barrier(0);
@@ -704,13 +750,15 @@ void gemm_tiled_kernel(GemmParams p) {
       if (pp + 1 < NP) convert_and_write(pp + 1);  // under the latency of the reads above
       __builtin_amdgcn_sched_barrier(0);
       const int n = n0 + wn * WTN + jp * PASS_J * 32 + rd_col;
+      // (a lane whose columns lie past N is sent past the extent: its stores are dropped)
+      const uint32_t c_lane_pass = n < p.N ? c_lane : 0x80000000u;
 #pragma unroll
       for (int it = 0; it < ITERS; ++it) {
         const int r = it * ROWS_PER_READ + rd_row;
         const v4i out = rows16[it];
-        if (ALIGNED) {
+        if (VECTOR) {
           // lane part (rd_row, rd_col) + scalar part (block row, read round, pass column)
-          store_chunk_streaming(out, c_rsrc, c_lane,
+          store_chunk_streaming(out, c_rsrc, c_lane_pass,
                                 (uint32_t)(i * 32 + it * ROWS_PER_READ) * c_row_bytes + (uint32_t)(jp * PASS_J * 32 * 2));
         } else {
           const int m = m0 + wm * WTM + i * 32 + r;
@@ -897,14 +945,11 @@ void gemm_tiled_kernel(GemmParams p) {
       } else {
         // sb already names the next step's stage; the one before it held this tile's last step
         uint8_t* free_b = lds + LDS_B0 + ((sb + kStagesB - 1) % kStagesB) * STAGE_B;
-        const bool interior = (loc.m0 + BM <= loc.m_end) && (loc.n0 + BN <= p.N);
-        // the vector epilogue stores 16 bytes of C and reads b_scale 16 and bias 8 bytes at a time
-        // (a group's slice of b_scale must start aligned too); anything else takes the scalar one
-        const uintptr_t bits = reinterpret_cast<uintptr_t>(p.c) | (uintptr_t)(p.ldc * 2) |
-                               reinterpret_cast<uintptr_t>(p.b_scale) | (reinterpret_cast<uintptr_t>(p.bias) << 1) |
-                               (GROUPED ? (uintptr_t)(p.N * 4) : 0);
+        // 16-byte stores need C's base and row pitch aligned and N a multiple of 8 (no lane's 8 columns
+        // straddle the edge); anything else stores element by element
+        const uintptr_t bits = reinterpret_cast<uintptr_t>(p.c) | (uintptr_t)(p.ldc * 2) | (uintptr_t)(p.N * 2);
         // (the output type is a compile-time property of the epilogue code: one uniform branch per tile)
-        if (interior && (bits & 15) == 0) {
+        if ((bits & 15) == 0) {
           if (p.out_f16) epilogue(loc, std::true_type{}, std::true_type{}, free_b);
           else epilogue(loc, std::true_type{}, std::false_type{}, free_b);
         } else {
