@@ -200,6 +200,13 @@ __device__ __forceinline__ uint16_t load_u16_checked(__amdgpu_buffer_rsrc_t rsrc
 #endif
 }
 
+// Range-checked store of 4 floats per lane through a buffer descriptor (dropped past the extent).
+__device__ __forceinline__ void store_f32x4_checked(v4f data, __amdgpu_buffer_rsrc_t rsrc, uint32_t lane_off, uint32_t wave_off) {
+#if defined(__HIP_DEVICE_COMPILE__)
+  __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(v4i, data), rsrc, (int)lane_off, (int)wave_off, 0);
+#endif
+}
+
 // One wave-wide streaming store of 16 bytes per lane through a buffer descriptor (address = base +
 // lane_off + wave_off): the output is written once and read by a later kernel at best.
 __device__ __forceinline__ void store_chunk_streaming(v4i data, __amdgpu_buffer_rsrc_t rsrc, uint32_t lane_off,
@@ -641,9 +648,11 @@ void gemm_tiled_kernel(GemmParams p) {
     // The lane-dependent addresses below are the same for every tile; derived from an opaque
     // copy of the lane id they are recomputed here (a few integer operations) instead of
     // being hoisted out of the tile loop, where they would occupy registers through the K loop.
-    // (the lane id itself comes from the hardware's lane count, so not even it stays live)
-    int lane_e = (int)__builtin_amdgcn_mbcnt_hi(~0u, __builtin_amdgcn_mbcnt_lo(~0u, 0u));
-    asm volatile("" : "+v"(lane_e));
+    // (the lane id itself comes from the hardware's lane count, inside the opaque statement: as a
+    // loop invariant it would be moved in front of the K loop and, with no register to spare there,
+    // spilled; its reload at this point waits for every load in flight)
+    int lane_e;
+    asm volatile("v_mbcnt_lo_u32_b32 %0, -1, 0\n\tv_mbcnt_hi_u32_b32 %0, -1, %0" : "=v"(lane_e));
     const int l32 = lane_e & 31, half = lane_e >> 5;
     const int wr_key = key(l32);
     const int wr_half = half * 8;  // where this lane's 8 bytes sit inside a chunk
@@ -774,29 +783,49 @@ void gemm_tiled_kernel(GemmParams p) {
     __builtin_amdgcn_sched_barrier(0);
   };
 
-  // ---- split-K: raw fp32 partial sums of this item to partial[split][m][n] (same lane layout
-  // as the epilogue: 4 consecutive n per lane, one 16-byte store when aligned)
+  // ---- split-K: raw fp32 partial sums of this item to partial[split][m][n]: the lane layout the
+  // MFMA leaves (4 consecutive n per lane), one 16-byte buffer store per 4 values when N is a multiple
+  // of 4: rows past M fall outside the descriptor's extent, lanes past N are sent there, and the
+  // values go from the accumulators to memory without passing through other registers.
   auto store_partial = [&](int m0, int n0, int split) {
+    int lane_e;  // (inside the opaque statement for the reason given in the epilogue)
+    asm volatile("v_mbcnt_lo_u32_b32 %0, -1, 0\n\tv_mbcnt_hi_u32_b32 %0, -1, %0" : "=v"(lane_e));
+    const int l32 = lane_e & 31, half = lane_e >> 5;
     float* base = p.partial + (size_t)split * p.M * p.N;
-    const bool vec = (p.N & 3) == 0;
-#pragma unroll
-    for (int i = 0; i < MT; ++i) {
-      const int m = m0 + wm * WTM + i * 32 + l32;
+    if ((p.N & 3) == 0) {
+      const uint32_t row_bytes = (uint32_t)p.N * 4u;  // (N*4*128 < 2^31 by the host's check of the workspace plan)
+      const int rows = min(max(p.M - (m0 + wm * WTM), 0), WTM);
+      const __amdgpu_buffer_rsrc_t rsrc = __builtin_amdgcn_make_buffer_rsrc(
+          base + ((size_t)(m0 + wm * WTM) * p.N + n0 + wn * WTN), 0, (int)((uint32_t)rows * row_bytes), 0x00020000);
+      const uint32_t lane_off = (uint32_t)l32 * row_bytes + (uint32_t)(4 * half) * 4u;
 #pragma unroll
       for (int j = 0; j < NT; ++j) {
-        __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
         for (int q = 0; q < 4; ++q) {
           const int n = n0 + wn * WTN + j * 32 + 8 * q + 4 * half;
-          const v4f v = {acc[i][j][4 * q], acc[i][j][4 * q + 1], acc[i][j][4 * q + 2], acc[i][j][4 * q + 3]};
-          if (m < p.M) {
-            float* dst = base + (size_t)m * p.N + n;
-            if (vec && n + 3 < p.N) {
-              *(v4f*)dst = v;
-            } else {
+          const uint32_t lo = n < p.N ? lane_off : 0x80000000u;
+#pragma unroll
+          for (int i = 0; i < MT; ++i) {
+            const v4f v = {acc[i][j][4 * q], acc[i][j][4 * q + 1], acc[i][j][4 * q + 2], acc[i][j][4 * q + 3]};
+            store_f32x4_checked(v, rsrc, lo, (uint32_t)(i * 32) * row_bytes + (uint32_t)(j * 32 + 8 * q) * 4u);
+          }
+        }
+      }
+    } else {
+#pragma unroll
+      for (int i = 0; i < MT; ++i) {
+        const int m = m0 + wm * WTM + i * 32 + l32;
+#pragma unroll
+        for (int j = 0; j < NT; ++j) {
+          __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+          for (int q = 0; q < 4; ++q) {
+            const int n = n0 + wn * WTN + j * 32 + 8 * q + 4 * half;
+            if (m < p.M) {
+              float* dst = base + (size_t)m * p.N + n;
 #pragma unroll
               for (int e = 0; e < 4; ++e)
-                if (n + e < p.N) dst[e] = v[e];
+                if (n + e < p.N) dst[e] = acc[i][j][4 * q + e];
             }
           }
         }
@@ -2060,6 +2089,8 @@ int mi355x_fp8_rowwise_gemm_ex(const void* a, const void* b, const float* a_scal
                         plan.splits, need, workspace ? workspace_bytes : (size_t)0);
           plan = plan_from_variant(M, N, K, plan_bits, 1);
         }
+        // (the partial sums of a tile are addressed with 32-bit byte offsets that must stay below 2^31)
+        if (plan.splits > 1 && N * 512 > (int64_t)INT32_MAX) plan = plan_from_variant(M, N, K, plan_bits & 0xff00, 1);
         if (plan.splits > 1 && (reinterpret_cast<uintptr_t>(workspace) & 15))
           return fail(MI355X_FP8_EINVAL, "workspace must be 16-byte aligned");
         p.splits = plan.splits;
