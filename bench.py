@@ -222,6 +222,25 @@ def time_quantiser(r, k, dtype, dev, steps=60, copies=3):
     return dict(us=ms * 1e3, gbps=nbytes / ms / 1e6, bound="hbm", frac=nbytes / ms / 1e6 / PEAK_HBM_GBPS)
 
 
+def time_fused_front_end(which, r, k, dev, steps=60, copies=3):
+    """Fused front ends (RMSNorm or SiLU-mul, then the row-wise quantiser, one kernel): algorithmic
+    bytes = the bf16 source row(s) + fp8 output + one f32 scale per row (the RMSNorm weight vector is
+    shared by all rows and stays in cache); sources rotate."""
+    from tritonbench_amd import ops
+
+    g = _generator(dev, r, k, 5)
+    x1 = [torch.randn((r, k), generator=g, device=dev, dtype=torch.float32).to(torch.bfloat16) for _ in range(copies)]
+    if which == "rmsnorm":
+        w = torch.randn((k,), generator=g, device=dev, dtype=torch.float32).to(torch.bfloat16)
+        ms = timed_calls(lambda i: ops.rms_norm_fp8_rowwise_quant(x1[i % copies], w), steps)
+        nbytes = r * k * 3 + 4 * r + 2 * k
+    else:
+        x2 = [torch.randn((r, k), generator=g, device=dev, dtype=torch.float32).to(torch.bfloat16) for _ in range(copies)]
+        ms = timed_calls(lambda i: ops.silu_mul_fp8_rowwise_quant(x1[i % copies], x2[i % copies]), steps)
+        nbytes = r * k * 5 + 4 * r
+    return dict(us=ms * 1e3, gbps=nbytes / ms / 1e6, bound="hbm", frac=nbytes / ms / 1e6 / PEAK_HBM_GBPS)
+
+
 def time_grouped(g, m, n, k, dev, steps=40, copies=2):
     """Grouped form (equal groups, as the reference's input generator makes them):
     flops = 2*M*N*K, bytes = M*K + G*N*K + 2*M*N."""
@@ -438,6 +457,8 @@ def main():
         configs["quantise_f32_8192x8192"] = time_quantiser(8192, 8192, torch.float32, dev)
         configs["quantise_bf16_8192x8192"] = time_quantiser(8192, 8192, torch.bfloat16, dev)
         configs["quantise_bf16_57344x8192"] = time_quantiser(57344, 8192, torch.bfloat16, dev, steps=20, copies=2)
+        configs["rmsnorm_quantise_bf16_8192x8192"] = time_fused_front_end("rmsnorm", 8192, 8192, dev)
+        configs["silu_mul_quantise_bf16_8192x8192"] = time_fused_front_end("silu_mul", 8192, 8192, dev)
         line["configs"] = configs
 
     if not args.no_cpu_baseline:

@@ -221,6 +221,32 @@ int mi355x_fp8_rowwise_quantize(const void* x, int src_type,
                                 int64_t R, int64_t K, int64_t ldx, int64_t ldq,
                                 void* stream);
 
+/*
+ * Fused front ends: normalise or gate the bf16 activation and quantise it row-wise in one pass
+ * (the row is read once; only the e4m3fn codes and one f32 scale per row are written). They stand
+ * in for rms_norm_fp8_rowwise_quant(x1, wd) and silu_mul_fp8_rowwise_quant(x1, x2) in the timed
+ * callables of tritonbench/operators/fp8_fused_quant_gemm_rowwise/operator.py:86-94 and :111-119
+ * (those kernels live outside the reference repository; the arithmetic below is this library's):
+ *
+ *   RMSNorm    y[r,k] = (x[r,k] * rstd[r]) * weight[k],   rstd[r] = 1 / sqrt(mean_k x[r,k]^2 + eps)
+ *   SiLU-mul   y[r,k] = (x1[r,k] / (1 + exp(-x1[r,k]))) * x2[r,k]
+ *
+ * all in f32 on the bf16 inputs, followed by the row-wise quantiser's arithmetic on y as on an
+ * f32 tensor (see mi355x_fp8_rowwise_quantize): xq, inv_scale feed mi355x_fp8_rowwise_gemm.
+ *
+ *   x, x1, x2  bf16 [R, K], row strides ldx / ldx1 / ldx2 (elements, multiples of 8)
+ *   weight     bf16 [K]                    xq  e4m3fn [R, K], row stride ldq (multiple of 16)
+ *   K a multiple of 8; x, x1, x2, weight and xq 16-byte aligned; eps >= 0.
+ */
+int mi355x_fp8_rmsnorm_rowwise_quantize(const void* x, const void* weight, float eps,
+                                        void* xq, float* inv_scale,
+                                        int64_t R, int64_t K, int64_t ldx, int64_t ldq,
+                                        void* stream);
+int mi355x_fp8_silu_mul_rowwise_quantize(const void* x1, const void* x2,
+                                         void* xq, float* inv_scale,
+                                         int64_t R, int64_t K, int64_t ldx1, int64_t ldx2, int64_t ldq,
+                                         void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -13,6 +13,17 @@ What is restated, and from where (paths relative to the tritonbench checkout):
   make_inputs           operator.py:280-297 (shapes, per-row A and per-row-of-[N,K] B
                         quantisation, optional bf16 bias), seeded as utils/env_utils.py:20
 
+  rms_norm / silu_mul / *_fp8_rowwise_quant
+                        the front ends of tritonbench/operators/fp8_fused_quant_gemm_rowwise/
+                        operator.py:86-131. The kernels that operator times (rms_norm,
+                        rms_norm_fp8_rowwise_quant, silu_mul, silu_mul_fp8_rowwise_quant) are
+                        imported from `gen_ai.llm_inference.fb.llm.kernel`, which is not part of the
+                        checkout, so the published definitions are restated: RMSNorm
+                        y = x * rsqrt(mean(x^2) + eps) * w and SwiGLU's SiLU(x1) * x2, evaluated in
+                        fp32 on the bf16 inputs, followed by fp8_row_quantize on the fp32 result.
+                        Parity unpinned for what those definitions leave open: the default eps, the
+                        order of the two multiplications and any bf16 rounding inside the absent kernels.
+
 How each function is pinned (tests/test_oracle_*.py):
   fp8_row_quantize      against an independent numpy restatement built on the bit-level
                         codec of oracle/e4m3.py, against oracle/fp8_rowwise_ref.c, and through
@@ -21,6 +32,9 @@ How each function is pinned (tests/test_oracle_*.py):
   dequant_matmul        against float64 brute force (gemm_f64, numpy) on small and ragged
                         shapes, bit-exact integer cases, identity / one-hot operands, and
                         oracle/fp8_rowwise_ref.c
+  rms_norm              against torch.nn.functional.rms_norm, a float64 loop over small rows, scale
+                        invariance at eps = 0 and the constant-row closed form
+  silu_mul              against torch.nn.functional.silu and the float64 definition
   matmul_fp8_row's own rounding / accumulation order and f8f8bf16_rowwise's CK instance
   are NOT reproducible without FBGEMM: parity unpinned for those (the tolerance
   rtol 1e-2 / atol 1e-2 is what absorbs them).
@@ -260,3 +274,40 @@ CONFIGS = {
     ),
     "c5_ragged_bias": dict(shapes=[(1000, 3000, 4112), (4097, 7168, 2048)], sigma=1.0, bias=True),
 }
+
+
+def rms_norm(x: torch.Tensor, weight: torch.Tensor, eps: float = 1e-5) -> torch.Tensor:
+    """RMSNorm with a weight vector in fp32: (x * rstd) * w, rstd = 1/sqrt(mean(x^2) + eps) with the
+    mean taken in float64 and rounded once (the front end of operator.py:86-109 of
+    fp8_fused_quant_gemm_rowwise; the kernel there is not in the checkout)."""
+    xf = x.to(torch.float32)
+    ms = xf.to(torch.float64).pow(2).mean(dim=1)
+    rstd = (1.0 / torch.sqrt(ms + eps)).to(torch.float32)
+    return (xf * rstd[:, None]) * weight.to(torch.float32)[None, :]
+
+
+def silu_mul(x1: torch.Tensor, x2: torch.Tensor) -> torch.Tensor:
+    """SiLU(x1) * x2 in fp32 (operator.py:111-131 of fp8_fused_quant_gemm_rowwise)."""
+    a = x1.to(torch.float32)
+    return (a / (1.0 + torch.exp(-a))) * x2.to(torch.float32)
+
+
+def rms_norm_fp8_rowwise_quant(x, weight, eps: float = 1e-5):
+    """(xq, inverse scale) of the normalised activation, quantised as an fp32 tensor."""
+    return fp8_row_quantize(rms_norm(x, weight, eps))
+
+
+def silu_mul_fp8_rowwise_quant(x1, x2):
+    return fp8_row_quantize(silu_mul(x1, x2))
+
+
+def make_fused_inputs(m: int, n: int, k: int, seed_tag: int = 0):
+    """x1, x2 [m,k], w [n,k], wd [k] as bf16 standard normals (get_input_iter of
+    fp8_fused_quant_gemm_rowwise/operator.py:154-165), plus the quantised weight."""
+    g = torch.Generator().manual_seed(_sub_seed(m, n, k, f"fused{seed_tag}"))
+    x1 = torch.randn((m, k), generator=g).to(torch.bfloat16)
+    x2 = torch.randn((m, k), generator=g).to(torch.bfloat16)
+    w = torch.randn((n, k), generator=g).to(torch.bfloat16)
+    wd = torch.randn((k,), generator=g).to(torch.bfloat16)
+    wq, w_scale = fp8_row_quantize(w)
+    return x1, x2, wq, w_scale, wd

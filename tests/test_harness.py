@@ -453,3 +453,35 @@ def test_cuda_time_metric_on_the_gpu(gpu_device):
     dev = table[0][headers.index("hip_mi355x-cuda_time")]
     # a split-K plan: two kernels per call, operands evicted before each, no launch gaps counted
     assert 0.010 < dev.p50 < 0.100 and 0.010 < lat.p50 < 0.100
+
+
+def test_fused_quant_operator_cpu_plumbing():
+    from oracle import fp8_rowwise as orc
+    from tritonbench_amd.harness.loader import list_operators, load_opbench_by_name
+    from tritonbench_amd.operators.fp8_fused_quant_gemm_rowwise import operator as fq
+
+    assert "fp8_fused_quant_gemm_rowwise" in list_operators()
+    assert len(fq.BUILDIN_SHAPES) == 20 and fq.BUILDIN_SHAPES[0] == (1, 2304, 2048) and fq.BUILDIN_SHAPES[-1] == (16384, 8192, 13312)
+    Op = load_opbench_by_name("fp8_fused_quant_gemm_rowwise")
+    args, extra = get_parser().parse_known_args(
+        ["--op", "fp8_fused_quant_gemm_rowwise", "--device", "cpu", "--m", "5", "--n", "48", "--k", "272",
+         "--metrics", "latency,tflops", "--only", "_rms_norm_dequant_cpu"])
+    op = Op(tb_args=args, extra_args=extra)
+    x1, x2, wq, w_scale, wd = next(op.get_input_iter())
+    assert x1.dtype == torch.bfloat16 and x1.shape == (5, 272) and x2.shape == (5, 272)
+    assert wq.shape == (48, 272) and w_scale.shape == (48,) and wd.shape == (272,)
+    # the operator's CPU chain is the oracle's: front end, row quantiser, dequantised product
+    xq, xs = orc.rms_norm_fp8_rowwise_quant(x1, wd, fq.RMS_NORM_EPS)
+    want = orc.dequant_matmul(xq, wq, xs, w_scale, None)
+    # (a code that falls the other way on a rounding tie moves single terms of the sums by one e4m3 step)
+    got = op._rms_norm_dequant_cpu(x1, x2, wq, w_scale, wd)().double()
+    assert (got - want.double()).norm() / want.double().norm() <= 1e-2
+    op.run(1, 2)
+    headers, table = op.output._table()
+    assert headers == ["(M, N, K)", "rms_norm_cpu_ref-latency", "rms_norm_cpu_ref-tflops"]
+    assert table[0][0] == (5, 48, 272)
+    assert table[0][2] == pytest.approx(2 * 5 * 48 * 272 / table[0][1].p50 / 1e12 * 1e3)
+    for name in ("rms_norm_fused", "rms_norm_quant", "silu_mul_fused", "silu_mul_quant"):
+        assert name in REGISTERED_BENCHMARKS["fp8_fused_quant_gemm_rowwise"]
+    with pytest.raises((RuntimeError, NotImplementedError)):
+        op.rms_norm_fused(x1, x2, wq, w_scale, wd)()

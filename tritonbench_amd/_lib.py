@@ -81,6 +81,14 @@ SIGNATURES = {
         c_int,
         [c_void_p, c_int, c_void_p, c_void_p, c_int64, c_int64, c_int64, c_int64, c_void_p],
     ),
+    "mi355x_fp8_rmsnorm_rowwise_quantize": (
+        c_int,
+        [c_void_p, c_void_p, ctypes.c_float, c_void_p, c_void_p, c_int64, c_int64, c_int64, c_int64, c_void_p],
+    ),
+    "mi355x_fp8_silu_mul_rowwise_quantize": (
+        c_int,
+        [c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int64, c_int64, c_int64, c_void_p],
+    ),
 }
 
 _lock = threading.Lock()

@@ -1682,6 +1682,165 @@ __global__ __launch_bounds__(THREADS) void quantize_rows_vec_kernel(const SrcT* 
   for (int c = tid + THREADS * CACHE; c < nchunks; c += THREADS) convert_store(xr[c], c);
 }
 
+
+// ------------------------------------------------------------------------------------
+// Fused front ends of the row-wise GEMM: the activation is normalised (RMSNorm with a weight
+// vector) or gated (SiLU(x1) * x2) and quantised row-wise in one pass, so the bf16 row is read
+// from memory once and nothing but the e4m3fn codes and one scale per row is written.
+// One workgroup per row; a lane keeps the fp32 values of up to CACHE 16-byte chunks (8 bf16
+// each) in registers across the passes: [sum of squares ->] value and row maximum -> convert.
+// Rows longer than THREADS*CACHE chunks re-read and recompute the rest. All arithmetic is fp32:
+//   RMSNorm   y = (x * rstd) * w,  rstd = 1 / sqrt(mean(x^2) + eps)
+//   SiLU-mul  y = (x1 / (1 + exp(-x1))) * x2
+// then the quantiser's arithmetic on y as on an fp32 tensor (row_scale<float>, clamp, RNE).
+// ------------------------------------------------------------------------------------
+constexpr int kFusedRmsNorm = 0, kFusedSiluMul = 1;
+
+template <int OP, int CACHE, int THREADS>
+__global__ __launch_bounds__(THREADS) void fused_rowwise_quant_kernel(const uint16_t* x1, const uint16_t* x2,
+                                                                      float eps, uint8_t* xq, float* inv_scale,
+                                                                      int K, long ld1, long ld2, long ldq) {
+  using V = VecTraits<uint16_t>;
+  constexpr int EPV = 8;
+  __shared__ float wave_part[THREADS / 64];
+  const long row = blockIdx.x;
+  const v4i* r1 = (const v4i*)(x1 + row * ld1);
+  // RMSNorm: the weight vector, shared by all rows; SiLU-mul: the row of the second operand
+  const v4i* r2 = (const v4i*)(OP == kFusedRmsNorm ? x2 : x2 + row * ld2);
+  uint8_t* qr = xq + row * ldq;
+  const int nchunks = K / EPV;
+  const int tid = threadIdx.x;
+
+  // sums (or maxima) of one value per lane over the workgroup; every lane gets the result
+  auto block_reduce = [&](float v, auto op) -> float {
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) v = op(v, __shfl_xor(v, o));
+    __syncthreads();  // the previous round's readers are done
+    if ((tid & 63) == 0) wave_part[tid >> 6] = v;
+    __syncthreads();
+    float r = wave_part[0];
+#pragma unroll
+    for (int w = 1; w < THREADS / 64; ++w) r = op(r, wave_part[w]);
+    return r;
+  };
+  // (hardware exponential and reciprocal, about one ulp each: the result is rounded to 4 significant
+  // bits next; the library forms cost six times the instructions and made the kernel compute-bound)
+  auto silu_mul = [](float a, float b) -> float { return (a * __frcp_rn(1.0f + __expf(-a))) * b; };
+
+  float vals[CACHE][EPV];
+  float rstd = 0.0f;
+  if (OP == kFusedRmsNorm) {
+    // pass 1: x to registers, sum of squares (lanes past the row's end re-read the last chunk and
+    // leave it out of the sum)
+    float ss = 0.0f;
+#pragma unroll
+    for (int i = 0; i < CACHE; ++i) {
+      const int c = tid + THREADS * i;
+      V::unpack(__builtin_nontemporal_load(r1 + min(c, nchunks - 1)), vals[i]);
+      if (c < nchunks) {
+#pragma unroll
+        for (int e = 0; e < EPV; ++e) ss = __builtin_fmaf(vals[i][e], vals[i][e], ss);
+      }
+    }
+    for (int c = tid + THREADS * CACHE; c < nchunks; c += THREADS) {
+      float f[EPV];
+      V::unpack(r1[c], f);
+#pragma unroll
+      for (int e = 0; e < EPV; ++e) ss = __builtin_fmaf(f[e], f[e], ss);
+    }
+    ss = block_reduce(ss, [](float a, float b) { return a + b; });
+    rstd = 1.0f / sqrtf(ss / (float)K + eps);
+  }
+  // value of chunk c from its raw operands
+  auto value = [&](const float (&a)[EPV], const float (&b)[EPV], float (&y)[EPV]) {
+#pragma unroll
+    for (int e = 0; e < EPV; ++e) y[e] = OP == kFusedRmsNorm ? (a[e] * rstd) * b[e] : silu_mul(a[e], b[e]);
+  };
+  // pass 2: values (kept for the cached chunks) and the row's absolute maximum
+  float amax = 0.0f;
+#pragma unroll
+  for (int i = 0; i < CACHE; ++i) {
+    const int c = min(tid + THREADS * i, nchunks - 1);
+    float a[EPV], b[EPV];
+    if (OP == kFusedRmsNorm) {
+#pragma unroll
+      for (int e = 0; e < EPV; ++e) a[e] = vals[i][e];
+    } else {
+      V::unpack(__builtin_nontemporal_load(r1 + c), a);
+    }
+    V::unpack(OP == kFusedRmsNorm ? r2[c] : __builtin_nontemporal_load(r2 + c), b);
+    value(a, b, vals[i]);
+#pragma unroll
+    for (int e = 0; e < EPV; ++e) amax = max_keep_nan(amax, fabsf(vals[i][e]));
+  }
+  for (int c = tid + THREADS * CACHE; c < nchunks; c += THREADS) {
+    float a[EPV], b[EPV], y[EPV];
+    V::unpack(r1[c], a);
+    V::unpack(r2[c], b);
+    value(a, b, y);
+#pragma unroll
+    for (int e = 0; e < EPV; ++e) amax = max_keep_nan(amax, fabsf(y[e]));
+  }
+  amax = block_reduce(amax, [](float a, float b) { return max_keep_nan(a, b); });
+
+  const float scale = row_scale<float>(amax);
+  if (tid == 0) inv_scale[row] = 1.0f / scale;
+  const bool finite_row = amax < __builtin_inff();  // a NaN or an infinity takes the integer encoder, which carries NaN through
+  auto convert_store = [&](const float (&y)[EPV], int c) {
+    if (finite_row) {
+      float f[EPV];
+#pragma unroll
+      for (int e = 0; e < EPV; ++e) f[e] = fminf(fmaxf(y[e] * scale, -448.0f), 448.0f);
+      int lo = __builtin_amdgcn_cvt_pk_fp8_f32(f[0], f[1], 0, false);
+      lo = __builtin_amdgcn_cvt_pk_fp8_f32(f[2], f[3], lo, true);
+      int hi = __builtin_amdgcn_cvt_pk_fp8_f32(f[4], f[5], 0, false);
+      hi = __builtin_amdgcn_cvt_pk_fp8_f32(f[6], f[7], hi, true);
+      *(v2u*)(qr + (size_t)c * 8) = (v2u){(uint32_t)lo, (uint32_t)hi};
+    } else {
+#pragma unroll
+      for (int e = 0; e < EPV; ++e) qr[(size_t)c * 8 + e] = quantize_one<float>(y[e], scale);
+    }
+  };
+  // pass 3: convert. Two consecutive rounds of cached chunks meet in a wave-private LDS strip and
+  // leave as one 16-byte store per lane (LDS executes a wave's operations in order: no barrier).
+  __shared__ __attribute__((aligned(16))) uint8_t strip[THREADS / 64][1024];
+  uint8_t* mine = strip[tid >> 6];
+  const int lane = tid & 63;
+  static_assert(CACHE % 2 == 0, "cached rounds are stored in pairs");
+#pragma unroll
+  for (int i0 = 0; i0 < CACHE; i0 += 2) {
+    if (finite_row && THREADS * (i0 + 2) <= nchunks) {  // uniform: every lane of every wave has both rounds
+#pragma unroll
+      for (int b = 0; b < 2; ++b) {
+        float f[EPV];
+#pragma unroll
+        for (int e = 0; e < EPV; ++e) f[e] = fminf(fmaxf(vals[i0 + b][e] * scale, -448.0f), 448.0f);
+        int lo = __builtin_amdgcn_cvt_pk_fp8_f32(f[0], f[1], 0, false);
+        lo = __builtin_amdgcn_cvt_pk_fp8_f32(f[2], f[3], lo, true);
+        int hi = __builtin_amdgcn_cvt_pk_fp8_f32(f[4], f[5], 0, false);
+        hi = __builtin_amdgcn_cvt_pk_fp8_f32(f[6], f[7], hi, true);
+        *(v2u*)(mine + b * 512 + lane * 8) = (v2u){(uint32_t)lo, (uint32_t)hi};
+      }
+      const int b = lane / 32, piece = lane % 32;
+      const v4i bytes = *(const v4i*)(mine + lane * 16);
+      *(v4i*)(qr + ((size_t)THREADS * (i0 + b) + (tid & ~63)) * EPV + piece * 16) = bytes;
+    } else {
+#pragma unroll
+      for (int b = 0; b < 2; ++b) {
+        const int c = tid + THREADS * (i0 + b);
+        if (c < nchunks) convert_store(vals[i0 + b], c);
+      }
+    }
+  }
+  for (int c = tid + THREADS * CACHE; c < nchunks; c += THREADS) {
+    float a[EPV], b[EPV], y[EPV];
+    V::unpack(r1[c], a);
+    V::unpack(r2[c], b);
+    value(a, b, y);
+    convert_store(y, c);
+  }
+}
+
 // ------------------------------------------------------------------------------------
 // Host side
 // ------------------------------------------------------------------------------------
@@ -2242,12 +2401,14 @@ int mi355x_fp8_rowwise_quantize(const void* x, int src_type, void* xq, float* in
   const bool vec = (reinterpret_cast<uintptr_t>(x) & 15) == 0 && (ldx * esz) % 16 == 0 && K % epv == 0 &&
                    (reinterpret_cast<uintptr_t>(xq) & 15) == 0 && ldq % 16 == 0;
   const bool long_row = K / epv > 8 * 256;  // more chunks than 256 lanes keep in registers
+  const bool short_row = K / epv <= 4 * 256;  // (bf16 source: half the registers, more workgroups per CU)
   if (vec && src_type == MI355X_FP8_SRC_F32) {
     auto kern = long_row ? quantize_rows_vec_kernel<float, 8, 1024> : quantize_rows_vec_kernel<float, 8, 256>;
     hipLaunchKernelGGL(kern, dim3((unsigned)R), dim3(long_row ? 1024 : 256), 0, s, (const float*)x,
                        (uint8_t*)xq, inv_scale, (int)K, (long)ldx, (long)ldq);
   } else if (vec && src_type == MI355X_FP8_SRC_BF16) {
-    auto kern = long_row ? quantize_rows_vec_kernel<uint16_t, 8, 1024> : quantize_rows_vec_kernel<uint16_t, 8, 256>;
+    auto kern = long_row ? quantize_rows_vec_kernel<uint16_t, 8, 1024>
+                         : short_row ? quantize_rows_vec_kernel<uint16_t, 4, 256> : quantize_rows_vec_kernel<uint16_t, 8, 256>;
     hipLaunchKernelGGL(kern, dim3((unsigned)R), dim3(long_row ? 1024 : 256), 0, s,
                        (const uint16_t*)x, (uint8_t*)xq, inv_scale, (int)K, (long)ldx, (long)ldq);
   } else if (src_type == MI355X_FP8_SRC_F32) {
@@ -2262,6 +2423,53 @@ int mi355x_fp8_rowwise_quantize(const void* x, int src_type, void* xq, float* in
   hipError_t e = hipGetLastError();
   if (e != hipSuccess) return fail(MI355X_FP8_ELAUNCH, "quantize kernel launch: %s", hipGetErrorString(e));
   return MI355X_FP8_OK;
+}
+
+namespace {
+int launch_fused_quant(int op, const void* x1, const void* x2, float eps, void* xq, float* inv_scale, int64_t R,
+                       int64_t K, int64_t ld1, int64_t ld2, int64_t ldq, void* stream) {
+  if (!x1 || !x2 || !xq || !inv_scale) return fail(MI355X_FP8_EINVAL, "null pointer");
+  if (R < 1 || K < 1 || ld1 < K || ldq < K || (op == kFusedSiluMul && ld2 < K))
+    return fail(MI355X_FP8_EINVAL, "bad shape or leading dimension");
+  if (R > INT32_MAX || K > INT32_MAX) return fail(MI355X_FP8_ENOTSUP, "dimension exceeds 2^31-1");
+  // whole 16-byte chunks of bf16, rows that start 16-byte aligned (the GEMM that follows wants K a
+  // multiple of 16 and 16-byte aligned rows of codes anyway)
+  if (K % 8 || ld1 % 8 || (op == kFusedSiluMul && ld2 % 8) || ldq % 16 || (reinterpret_cast<uintptr_t>(x1) & 15) ||
+      (reinterpret_cast<uintptr_t>(x2) & 15) || (reinterpret_cast<uintptr_t>(xq) & 15))
+    return fail(MI355X_FP8_ENOTSUP, "rows must hold whole 16-byte chunks and start 16-byte aligned");
+  if (!(eps >= 0.0f)) return fail(MI355X_FP8_EINVAL, "eps must be >= 0");
+  hipStream_t s = (hipStream_t)stream;
+  // chunks a lane keeps in registers: 4 for rows up to 8192 elements (half the registers, twice the
+  // workgroups per CU), 8 up to 16384, beyond that 1024 lanes per row
+  const int64_t chunks = K / 8;
+  const bool long_row = chunks > 8 * 256;
+  const bool short_row = chunks <= 4 * 256;
+  const dim3 grid((unsigned)R), block(long_row ? 1024 : 256);
+  const uint16_t* a = (const uint16_t*)x1;
+  const uint16_t* b = (const uint16_t*)x2;
+  if (op == kFusedRmsNorm) {
+    auto kern = long_row ? fused_rowwise_quant_kernel<kFusedRmsNorm, 8, 1024>
+                         : short_row ? fused_rowwise_quant_kernel<kFusedRmsNorm, 4, 256> : fused_rowwise_quant_kernel<kFusedRmsNorm, 8, 256>;
+    hipLaunchKernelGGL(kern, grid, block, 0, s, a, b, eps, (uint8_t*)xq, inv_scale, (int)K, (long)ld1, (long)ld2, (long)ldq);
+  } else {
+    auto kern = long_row ? fused_rowwise_quant_kernel<kFusedSiluMul, 8, 1024>
+                         : short_row ? fused_rowwise_quant_kernel<kFusedSiluMul, 4, 256> : fused_rowwise_quant_kernel<kFusedSiluMul, 8, 256>;
+    hipLaunchKernelGGL(kern, grid, block, 0, s, a, b, eps, (uint8_t*)xq, inv_scale, (int)K, (long)ld1, (long)ld2, (long)ldq);
+  }
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess) return fail(MI355X_FP8_ELAUNCH, "fused quantise kernel launch: %s", hipGetErrorString(e));
+  return MI355X_FP8_OK;
+}
+}  // namespace
+
+int mi355x_fp8_rmsnorm_rowwise_quantize(const void* x, const void* weight, float eps, void* xq, float* inv_scale,
+                                        int64_t R, int64_t K, int64_t ldx, int64_t ldq, void* stream) {
+  return launch_fused_quant(kFusedRmsNorm, x, weight, eps, xq, inv_scale, R, K, ldx, K, ldq, stream);
+}
+
+int mi355x_fp8_silu_mul_rowwise_quantize(const void* x1, const void* x2, void* xq, float* inv_scale, int64_t R,
+                                         int64_t K, int64_t ldx1, int64_t ldx2, int64_t ldq, void* stream) {
+  return launch_fused_quant(kFusedSiluMul, x1, x2, 0.0f, xq, inv_scale, R, K, ldx1, ldx2, ldq, stream);
 }
 
 }  // extern "C"

@@ -258,3 +258,50 @@ def fp8_row_quantize(x: torch.Tensor) -> Tuple[torch.Tensor, torch.Tensor]:
     )
     _lib.check(st, "mi355x_fp8_rowwise_quantize")
     return xq, inv_scale
+
+
+def _fused_quant_outputs(x: torch.Tensor) -> Tuple[torch.Tensor, torch.Tensor]:
+    r, k = x.shape
+    return (torch.empty((r, k), dtype=FP8_DTYPE, device=x.device),
+            torch.empty((r,), dtype=torch.float32, device=x.device))
+
+
+def rms_norm_fp8_rowwise_quant(x: torch.Tensor, weight: torch.Tensor, eps: float = 1e-5) -> Tuple[torch.Tensor, torch.Tensor]:
+    """RMSNorm with a weight vector and row-wise e4m3fn quantisation in one kernel; returns
+    (xq, inverse scale). Stands in for rms_norm_fp8_rowwise_quant(x1, wd) of
+    tritonbench/operators/fp8_fused_quant_gemm_rowwise/operator.py:86-94."""
+    lib = _lib.load()
+    _require_gpu(x, "x")
+    _require_gpu(weight, "weight")
+    if x.dim() != 2 or x.stride(1) != 1 or x.dtype != torch.bfloat16:
+        raise ValueError("x must be a 2-D bfloat16 tensor with unit column stride")
+    if weight.dtype != torch.bfloat16 or tuple(weight.shape) != (x.shape[1],) or weight.stride(0) != 1:
+        raise ValueError("weight must be a contiguous bfloat16 vector of length K")
+    xq, inv_scale = _fused_quant_outputs(x)
+    st = lib.mi355x_fp8_rmsnorm_rowwise_quantize(
+        x.data_ptr(), weight.data_ptr(), float(eps), xq.data_ptr(), inv_scale.data_ptr(),
+        x.shape[0], x.shape[1], x.stride(0), xq.stride(0), _stream_ptr(),
+    )
+    _lib.check(st, "mi355x_fp8_rmsnorm_rowwise_quantize")
+    return xq, inv_scale
+
+
+def silu_mul_fp8_rowwise_quant(x1: torch.Tensor, x2: torch.Tensor) -> Tuple[torch.Tensor, torch.Tensor]:
+    """SiLU(x1) * x2 and row-wise e4m3fn quantisation in one kernel; returns (xq, inverse scale).
+    Stands in for silu_mul_fp8_rowwise_quant(x1, x2) of
+    tritonbench/operators/fp8_fused_quant_gemm_rowwise/operator.py:111-119."""
+    lib = _lib.load()
+    _require_gpu(x1, "x1")
+    _require_gpu(x2, "x2")
+    for name, t in (("x1", x1), ("x2", x2)):
+        if t.dim() != 2 or t.stride(1) != 1 or t.dtype != torch.bfloat16:
+            raise ValueError(f"{name} must be a 2-D bfloat16 tensor with unit column stride")
+    if x1.shape != x2.shape:
+        raise ValueError("x1 and x2 must have the same shape")
+    xq, inv_scale = _fused_quant_outputs(x1)
+    st = lib.mi355x_fp8_silu_mul_rowwise_quantize(
+        x1.data_ptr(), x2.data_ptr(), xq.data_ptr(), inv_scale.data_ptr(),
+        x1.shape[0], x1.shape[1], x1.stride(0), x2.stride(0), xq.stride(0), _stream_ptr(),
+    )
+    _lib.check(st, "mi355x_fp8_silu_mul_rowwise_quantize")
+    return xq, inv_scale
