@@ -1,0 +1,68 @@
+"""The automatic choice of kernel family, tile configuration and split factor against the pinned
+alternatives, timed on the device: the cost estimates behind the choice are tables of measured
+constants, and a table that has drifted away from the kernels shows here as a choice that is
+clearly slower than one of its alternatives. Needs an MI355X.
+
+Timing: a captured graph of 16 launches over 4 rotating operand sets (cold weights, as a model's
+are), best of 4 replays after a warm-up replay. The bar is 12 %: the spread of repeated
+measurements of one plan on these shapes is 2-4 %."""
+import pytest
+import torch
+
+from tritonbench_amd import _lib, ops
+
+pytestmark = pytest.mark.gpu
+
+TOLERANCE = 1.12
+# decode- and small-prefill-sized rows of the Llama-3-70B projection sweep, and the small ragged shape with bias
+SHAPES = [(32, 8192, 8192, False), (64, 8192, 8192, False), (128, 8192, 8192, False), (128, 10240, 8192, False),
+          (32, 10240, 8192, False), (256, 8192, 8192, False), (1000, 3000, 4112, True)]
+
+
+def _time_us(dev, m, n, k, bias, variant, sets):
+    ws = ops.gemm_workspace(m, n, k, dev, variant)
+    stream = torch.cuda.Stream()
+    with torch.cuda.stream(stream):
+        def call(i):
+            xq, wq, xs, w_s, b, out = sets[i % len(sets)]
+            ops.fp8_gemm_rowwise(xq, wq, xs, w_s, bias=b, out=out, workspace=ws, variant=variant)
+        call(0)
+        torch.cuda.synchronize()
+        g = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g, stream=stream):
+            for i in range(16):
+                call(i)
+        g.replay()
+        torch.cuda.synchronize()
+        best = float("inf")
+        for _ in range(4):
+            start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            start.record(stream)
+            g.replay()
+            end.record(stream)
+            torch.cuda.synchronize()
+            best = min(best, start.elapsed_time(end) * 1e3 / 16)
+    return best
+
+
+@pytest.mark.parametrize("m,n,k,bias", SHAPES)
+def test_automatic_choice_is_close_to_the_best_alternative(gpu_device, m, n, k, bias):
+    print(f"case m={m} n={n} k={k} bias={bias}", flush=True)
+    dev = gpu_device
+    g = torch.Generator(device=dev).manual_seed(m + n + k)
+    sets = []
+    for _ in range(4):
+        xq, xs = ops.fp8_row_quantize(torch.randn((m, k), generator=g, device=dev))
+        wq, w_s = ops.fp8_row_quantize(torch.randn((n, k), generator=g, device=dev))
+        b = (0.1 * torch.randn((n,), generator=g, device=dev)).to(torch.bfloat16) if bias else None
+        sets.append((xq, wq, xs, w_s, b, torch.empty((m, n), dtype=torch.bfloat16, device=dev)))
+    alternatives = {f"tiled config {c}": _lib.tiled_variant(c, 0) for c in range(_lib.NUM_TILE_CONFIGS)}
+    if m <= 64:
+        alternatives["skinny"] = _lib.VARIANT_SKINNY
+        alternatives["skinny, one tile per workgroup"] = _lib.VARIANT_SKINNY | _lib.SKINNY_ONE_TILE
+    auto = _time_us(dev, m, n, k, bias, _lib.VARIANT_AUTO, sets)
+    times = {name: _time_us(dev, m, n, k, bias, v, sets) for name, v in alternatives.items()}
+    best_name = min(times, key=times.get)
+    print(f"  automatic {auto:.1f} us; " + ", ".join(f"{nm} {t:.1f}" for nm, t in times.items()), flush=True)
+    assert auto <= TOLERANCE * times[best_name], (
+        f"automatic choice takes {auto:.1f} us, '{best_name}' {times[best_name]:.1f} us: the cost tables need recalibrating")
