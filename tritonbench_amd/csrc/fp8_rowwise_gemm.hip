@@ -419,9 +419,16 @@ void gemm_tiled_kernel(GemmParams p) {
     // the pair into a three-operand median, which exists as a vector instruction only and would
     // pull the descriptor out of the scalar registers)
     const uint32_t extent = (uint32_t)min(rows_valid, rows_tile) * (uint32_t)ld;
+    // Base and extent are the same for every lane; they are pinned to scalar registers because a
+    // descriptor that the compiler takes for lane-dependent (the grouped form derives these from
+    // sizes it loads, through a clamp that only exists as a vector instruction) makes every load a
+    // loop over the distinct descriptors of the wave.
     OperandSrc o;
-    o.base = base;
-    o.extent = extent;
+    const uintptr_t b = reinterpret_cast<uintptr_t>(base);
+    o.base = reinterpret_cast<const uint8_t*>(
+        ((uintptr_t)(uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)(b >> 32)) << 32) |
+        (uintptr_t)(uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)b));
+    o.extent = (uint32_t)__builtin_amdgcn_readfirstlane((int)extent);
     o.wave_off = 8u * (uint32_t)wave * (uint32_t)ld;
     o.group_stride = 8u * NW * (uint32_t)ld;
     return o;
@@ -671,7 +678,7 @@ void gemm_tiled_kernel(GemmParams p) {
       sam[i] = BLOCKSCALE ? 1.0f : p.a_scale[min(m0 + wm * WTM + i * 32 + l32, loc.m_end - 1)];
     if (!BLOCKSCALE) {
       const int n_wave = n0 + wn * WTN;               // first column of the wave's tile
-      const int n_left = max(p.N - n_wave, 0);        // columns from there to the edge
+      const int n_left = __builtin_amdgcn_readfirstlane(max(p.N - n_wave, 0));  // columns from there to the edge
       const __amdgpu_buffer_rsrc_t s_rsrc = __builtin_amdgcn_make_buffer_rsrc(
           const_cast<float*>(p.b_scale) + ((GROUPED ? (size_t)loc.group * p.N : 0) + n_wave), 0, n_left * 4, 0x00020000);
       const __amdgpu_buffer_rsrc_t bias_rsrc = __builtin_amdgcn_make_buffer_rsrc(
@@ -738,7 +745,9 @@ void gemm_tiled_kernel(GemmParams p) {
     // The wave's part of the tile as a buffer: origin at its first element, extent = its valid rows
     // (none for a wave that lies past the edge); offsets stay below 2^31 by the host's check of ldc.
     const uint32_t c_row_bytes = (uint32_t)p.ldc * 2u;
-    const int c_rows = min(max(loc.m_end - (m0 + wm * WTM), 0), WTM);
+    // (pinned to a scalar register: the double clamp exists as a vector instruction only, and a
+    // descriptor held in vector registers makes every store a loop)
+    const int c_rows = __builtin_amdgcn_readfirstlane(min(max(loc.m_end - (m0 + wm * WTM), 0), WTM));
     const __amdgpu_buffer_rsrc_t c_rsrc = __builtin_amdgcn_make_buffer_rsrc(
         p.c + ((size_t)(m0 + wm * WTM) * p.ldc + n0 + wn * WTN), 0, (int)((uint32_t)c_rows * c_row_bytes), 0x00020000);
     const uint32_t c_lane = (uint32_t)rd_row * c_row_bytes + (uint32_t)rd_col * 2u;
@@ -794,7 +803,7 @@ void gemm_tiled_kernel(GemmParams p) {
     float* base = p.partial + (size_t)split * p.M * p.N;
     if ((p.N & 3) == 0) {
       const uint32_t row_bytes = (uint32_t)p.N * 4u;  // (N*4*128 < 2^31 by the host's check of the workspace plan)
-      const int rows = min(max(p.M - (m0 + wm * WTM), 0), WTM);
+      const int rows = __builtin_amdgcn_readfirstlane(min(max(p.M - (m0 + wm * WTM), 0), WTM));  // (scalar: see the epilogue)
       const __amdgpu_buffer_rsrc_t rsrc = __builtin_amdgcn_make_buffer_rsrc(
           base + ((size_t)(m0 + wm * WTM) * p.N + n0 + wn * WTN), 0, (int)((uint32_t)rows * row_bytes), 0x00020000);
       const uint32_t lane_off = (uint32_t)l32 * row_bytes + (uint32_t)(4 * half) * 4u;
