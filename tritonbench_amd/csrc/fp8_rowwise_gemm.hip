@@ -256,9 +256,9 @@ constexpr int kEpiPlain = 0, kEpiBias = 1, kEpiPartial = 2;
 constexpr size_t tiled_lds_bytes(int BM, int BN, int dist = kDefaultDist) {
   return (size_t)(dist * BM + (dist + 1) * BN) * kStepK;
 }
-// (the block-scaled form keeps a second accumulator set and needs the whole register file)
 constexpr int tiled_wgs_per_cu(int BM, int BN, bool blockscale = false, int dist = kDefaultDist) {
-  return !blockscale && tiled_lds_bytes(BM, BN, dist) <= 80 * 1024 ? 2 : 1;
+  (void)blockscale;
+  return tiled_lds_bytes(BM, BN, dist) <= 80 * 1024 ? 2 : 1;
 }
 
 //
@@ -268,8 +268,8 @@ constexpr int tiled_wgs_per_cu(int BM, int BN, bool blockscale = false, int dist
 // [ceil(M/128)][ceil(K/128)], b_scale [ceil(N/128)][ceil(K/128)], and every K step's product
 // is multiplied by a_scale[mb][kb] * b_scale[nb][kb] before it is added up. With wave tiles
 // inside one scale block and 128-byte steps that factor is one number per wave and step:
-// the MFMAs of a step go to a second accumulator set, which is folded into the first
-// (acc += s * tmp) behind the next step's MFMAs.
+// the accumulators are kept in units of the current step's factor (multiplied by the ratio of
+// consecutive factors in front of each step's MFMAs) and by the last factor in the epilogue.
 //
 // STREAM_B: the rows of B are fetched with the streaming cache policy. For launches with one or
 // two tile rows, where a panel of B is read by one or two workgroups and never again
@@ -537,36 +537,47 @@ void gemm_tiled_kernel(GemmParams p) {
   };
 
   v16f acc[MT][NT];  // defined by the first step of every work item
-  // BLOCKSCALE only: the running step's unscaled product, the factor it is waiting for, the
-  // K step the compute side is at, and the lane's share of the item's factors
-  // (sc[r] belongs to step 64*r + lane).
-  v16f tmp[BLOCKSCALE ? MT : 1][BLOCKSCALE ? NT : 1];
-  float s_pend = 0.0f;
+  // BLOCKSCALE only. The sum over K blocks of s_k * P_k (P_k the unscaled product of block k) is
+  // kept in units of the current block's factor: before step k adds P_k the accumulators are
+  // multiplied by s_(k-1) / s_k, and the epilogue multiplies by the last factor. One multiply per
+  // accumulator and step on the vector ALU, under the MFMAs' cover, and no second accumulator
+  // set: the kernel keeps the register budget of the plain 128x128 tile (two workgroups per CU).
+  // A factor of exactly zero is replaced by 2^-60 (its block then contributes P_k * 2^-60, nothing
+  // at the output's precision); factors are expected to span less than 2^60 within a row of blocks.
+  // Blocks 0 .. n-2 are rescaled in phase [B] of the step before (each under the cover of the next
+  // block's MFMA), the last one under the first MFMA of the step itself.
+  // s_pend / s_cur: the ratios to the next step / to this one; kt_c: the K step the compute side is
+  // at; the lane's share of the item's factors and ratios (sc[r], rt[r] belong to step 64*r + lane).
+  float s_pend = 1.0f, s_cur = 1.0f, s_last = 1.0f, n_pend = 1.0f, n_last = 1.0f;
   int kt_c = 0;
   constexpr int SC_REGS = 4;  // 256 steps = K up to 32768
-  float sc[SC_REGS] = {0.f, 0.f, 0.f, 0.f};
+  float sc[SC_REGS] = {0.f, 0.f, 0.f, 0.f}, rt[SC_REGS] = {1.f, 1.f, 1.f, 1.f};
   auto load_block_scales = [&](const TileLoc& loc) {
     // the scale block of this wave's tile (clamped for waves that lie past the matrix edge)
     const int mb = min(loc.m0 + wm * WTM, p.M - 1) / 128, nb = min(loc.n0 + wn * WTN, p.N - 1) / 128;
     const float* sa = p.a_scale + (size_t)mb * k_steps;
     const float* sb = p.b_scale + (size_t)nb * k_steps;
+    auto factor = [&](int kb) -> float {
+      const float f = sa[kb] * sb[kb];
+      return f == 0.0f ? 0x1p-60f : f;
+    };
 #pragma unroll
     for (int r = 0; r < SC_REGS; ++r) {
       const int kb = min(r * 64 + lane, k_steps - 1);
-      sc[r] = sa[kb] * sb[kb];
+      sc[r] = factor(kb);
+      rt[r] = kb > 0 ? factor(kb - 1) / sc[r] : 1.0f;
     }
   };
-  auto step_scale = [&](int kt) -> float {
+  auto lane_value = [&](const float (&regs)[SC_REGS], int kt) -> float {
     const int r = kt >> 6;
-    const float v = r == 0 ? sc[0] : r == 1 ? sc[1] : r == 2 ? sc[2] : sc[3];
+    const float v = r == 0 ? regs[0] : r == 1 ? regs[1] : r == 2 ? regs[2] : regs[3];
     return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), kt & 63));
   };
-  // folds block t of the waiting product into the accumulators (or starts them from zero)
-  auto fold_block = [&](int t, bool start) {
+  // brings block t of the accumulators from one step's factor to the next one's
+  auto fold_block = [&](int t, float ratio) {
     const int i = t / NT, j = t % NT;
-    auto& tm = tmp[BLOCKSCALE ? i : 0][BLOCKSCALE ? j : 0];
 #pragma unroll
-    for (int v = 0; v < 16; ++v) acc[i][j][v] = start ? 0.0f : __builtin_fmaf(s_pend, tm[v], acc[i][j][v]);
+    for (int v = 0; v < 16; ++v) acc[i][j][v] *= ratio;
   };
 
   // t-th MFMA of a half step (t = i*NT + j) on fragment set (fa, fb)
@@ -574,12 +585,7 @@ void gemm_tiled_kernel(GemmParams p) {
   auto mfma_one = [&](const Frag (&fa)[MT], const Frag (&fb)[NT], int t, bool fresh) {
     const int i = t / NT, j = t % NT;
     const v16f zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-    if (BLOCKSCALE) {
-      auto& tm = tmp[BLOCKSCALE ? i : 0][BLOCKSCALE ? j : 0];
-      tm = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(as_v8(fb[j]), as_v8(fa[i]), fresh ? zero : tm, 0, 0, 0, 0, 0, 0);
-    } else {
-      acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(as_v8(fb[j]), as_v8(fa[i]), fresh ? zero : acc[i][j], 0, 0, 0, 0, 0, 0);
-    }
+    acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(as_v8(fb[j]), as_v8(fa[i]), fresh ? zero : acc[i][j], 0, 0, 0, 0, 0, 0);
   };
   // u-th of the 2*(MT+NT) LDS reads that fill fragment set (fa, fb) with K half s
   auto read_one = [&](Frag (&fa)[MT], Frag (&fb)[NT], const uint8_t* rows_a, const uint8_t* rows_b, int s, int u) {
@@ -675,7 +681,7 @@ void gemm_tiled_kernel(GemmParams p) {
     us4 bv[HAS_BIAS ? NT : 1][4];
 #pragma unroll
     for (int i = 0; i < MT; ++i)
-      sam[i] = BLOCKSCALE ? 1.0f : p.a_scale[min(m0 + wm * WTM + i * 32 + l32, loc.m_end - 1)];
+      sam[i] = BLOCKSCALE ? s_last : p.a_scale[min(m0 + wm * WTM + i * 32 + l32, loc.m_end - 1)];
     if (!BLOCKSCALE) {
       const int n_wave = n0 + wn * WTN;               // first column of the wave's tile
       const int n_left = __builtin_amdgcn_readfirstlane(max(p.N - n_wave, 0));  // columns from there to the edge
@@ -883,6 +889,11 @@ void gemm_tiled_kernel(GemmParams p) {
   auto step = [&](auto first_tag, auto read_next_tag, auto plain_tag) {
     constexpr bool FIRST = decltype(first_tag)::value;
     constexpr bool READ_NEXT = decltype(read_next_tag)::value;
+    if (BLOCKSCALE) {  // (fetched from the lanes that hold them during the previous step, or at the item's start)
+      s_cur = s_pend;    // ratio that brought the accumulators to this step
+      s_pend = n_pend;   // ratio to the next step (applied in phase [B])
+      s_last = n_last;   // this step's factor: what the epilogue multiplies by after the last step
+    }
 
     // [A] MFMAs on x* (first K half of this step). Behind them, one per MFMA: the LDS reads
     //     of the second half (-> y*), and behind every other one a global->LDS load of
@@ -894,9 +905,10 @@ void gemm_tiled_kernel(GemmParams p) {
     __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
     for (int t = 0; t < NMFMA; ++t) {
-      if (BLOCKSCALE) fold_block(t, FIRST);  // the previous step's block t, before it is overwritten
-      mfma_one(xa, xb, t, BLOCKSCALE || FIRST);
+      mfma_one(xa, xb, t, FIRST);
       __builtin_amdgcn_sched_barrier(0);  // the MFMA goes first: what follows is issued under its cover
+      // (the last block of the previous step is brought to this step's units here, under the first MFMA's cover)
+      if (BLOCKSCALE && !FIRST && t == 0) fold_block(NMFMA - 1, s_cur);
 #pragma unroll
       for (int l = 0; l < B_GROUPS; ++l)
         if (l * NMFMA / B_GROUPS == t)
@@ -906,6 +918,10 @@ void gemm_tiled_kernel(GemmParams p) {
         if (u < NREAD) read_one(ya, yb, cur_a, cur_b, 1, u);
       if (t == B_LAST) advance_b(plain_tag);
       if (t == PREP_T) prepare_a_loads();
+      if (BLOCKSCALE && t == PREP_T) {
+        n_pend = lane_value(rt, min(kt_c + 2, k_steps - 1));
+        n_last = lane_value(sc, min(kt_c + 1, k_steps - 1));
+      }
       if (t == PREP_T2) {
         sa = (sa + 1 == kStagesA) ? 0 : sa + 1;
         sb = (sb + 1 == kStagesB) ? 0 : sb + 1;
@@ -928,6 +944,8 @@ void gemm_tiled_kernel(GemmParams p) {
     for (int t = 0; t < NMFMA; ++t) {
       mfma_one(ya, yb, t, false);
       __builtin_amdgcn_sched_barrier(0);
+      // block t-1 has had its last MFMA of this step: into the next step's units, under this MFMA's cover
+      if (BLOCKSCALE && READ_NEXT && t >= 1) fold_block(t - 1, s_pend);
 #pragma unroll
       for (int l = 0; l < A_GROUPS; ++l)
         if (l * NMFMA / A_GROUPS == t) load_group(std::false_type{}, a_src, ph_a.lane_off, ph_a.step_off, l, ph_a.stage);
@@ -942,7 +960,7 @@ void gemm_tiled_kernel(GemmParams p) {
       }
       __builtin_amdgcn_sched_barrier(0);
     }
-    if (BLOCKSCALE) s_pend = step_scale(kt_c++);
+    if (BLOCKSCALE) ++kt_c;
   };
   auto read_first_half = [&]() {
 #pragma unroll
@@ -960,6 +978,8 @@ void gemm_tiled_kernel(GemmParams p) {
     if (BLOCKSCALE) {
       load_block_scales(locate(walk_c, c_item));
       kt_c = split_begin(c_split);
+      n_pend = lane_value(rt, min(kt_c + 1, k_steps - 1));
+      n_last = lane_value(sc, kt_c);
     }
     if (n_steps == 1) {
       step(std::true_type{}, std::false_type{}, std::false_type{});
@@ -971,10 +991,6 @@ void gemm_tiled_kernel(GemmParams p) {
       for (; k < n_steps - DIST - 1; ++k) step(std::false_type{}, std::true_type{}, std::true_type{});
       for (; k < n_steps - 1; ++k) step(std::false_type{}, std::true_type{}, std::false_type{});
       step(std::false_type{}, std::false_type{}, std::false_type{});
-    }
-    if (BLOCKSCALE) {
-#pragma unroll
-      for (int t = 0; t < NMFMA; ++t) fold_block(t, false);  // the last step's product
     }
     {
       const TileLoc loc = locate(walk_c, c_item);
