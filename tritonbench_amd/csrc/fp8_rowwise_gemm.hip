@@ -43,7 +43,6 @@ typedef unsigned int v2u __attribute__((ext_vector_type(2)));
 
 constexpr int kNumXcd = 8;       // accelerator complex dies; workgroup ids round-robin over them
 constexpr int kNumCu = 256;
-constexpr int kBK = 128;         // bytes (= fp8 elements) of K one 16x16x128 MFMA consumes (skinny kernel step)
 constexpr int kChunk = 16;       // bytes moved per lane per load
 
 struct GemmParams {
@@ -1086,7 +1085,6 @@ template <int MT, int NTW, int DEPTH, int KW>
 __global__ __launch_bounds__(KW * 64) void gemm_skinny_kernel(GemmParams p) {
   constexpr int TILE = 16 * kStepK;                 // one 16-row operand tile of one step: 2 KB
   constexpr int NTILE = NTW + MT;                   // tiles per step: B tiles then A tiles
-  constexpr int LOADS = 2 * NTILE;                  // wave-wide loads per step
   constexpr int BUF = NTILE * TILE;                 // wave-private transpose buffer
   static_assert(NTW * MT * 1024 <= BUF, "the reduction reuses a wave's buffer for its partials");
 
@@ -1727,7 +1725,7 @@ __global__ __launch_bounds__(THREADS) void fused_rowwise_quant_kernel(const uint
                                                                       int K, long ld1, long ld2, long ldq) {
   using V = VecTraits<uint16_t>;
   constexpr int EPV = 8;
-  __shared__ float wave_part[THREADS / 64];
+  __shared__ float wave_part[2][THREADS / 64];  // one set per reduction: neither waits for the other's readers
   const long row = blockIdx.x;
   const v4i* r1 = (const v4i*)(x1 + row * ld1);
   // RMSNorm: the weight vector, shared by all rows; SiLU-mul: the row of the second operand
@@ -1737,27 +1735,35 @@ __global__ __launch_bounds__(THREADS) void fused_rowwise_quant_kernel(const uint
   const int tid = threadIdx.x;
 
   // sums (or maxima) of one value per lane over the workgroup; every lane gets the result
-  auto block_reduce = [&](float v, auto op) -> float {
+  auto block_reduce = [&](int set, float v, auto op) -> float {
 #pragma unroll
     for (int o = 32; o > 0; o >>= 1) v = op(v, __shfl_xor(v, o));
-    __syncthreads();  // the previous round's readers are done
-    if ((tid & 63) == 0) wave_part[tid >> 6] = v;
+    if ((tid & 63) == 0) wave_part[set][tid >> 6] = v;
     __syncthreads();
-    float r = wave_part[0];
+    float r = wave_part[set][0];
 #pragma unroll
-    for (int w = 1; w < THREADS / 64; ++w) r = op(r, wave_part[w]);
+    for (int w = 1; w < THREADS / 64; ++w) r = op(r, wave_part[set][w]);
     return r;
   };
   // (hardware exponential and reciprocal, about one ulp each: the result is rounded to 4 significant
-  // bits next; the library forms cost six times the instructions and made the kernel compute-bound)
-  auto silu_mul = [](float a, float b) -> float { return (a * __frcp_rn(1.0f + __expf(-a))) * b; };
+  // bits next; the library exponential costs six times the instructions and a correctly rounded
+  // quotient ten, which together made the kernel compute-bound)
+  auto silu_mul = [](float a, float b) -> float { return (a * __builtin_amdgcn_rcpf(1.0f + __expf(-a))) * b; };
 
   float vals[CACHE][EPV];
+  // (the 1024-lane form has 128 registers per lane and none to spare for them)
+  constexpr bool EARLY_WEIGHTS = OP == kFusedRmsNorm && THREADS <= 256;
+  v4i wts[EARLY_WEIGHTS ? CACHE : 1];
   float rstd = 0.0f;
   if (OP == kFusedRmsNorm) {
     // pass 1: x to registers, sum of squares (lanes past the row's end re-read the last chunk and
-    // leave it out of the sum)
+    // leave it out of the sum). The weights of the cached chunks are asked for here as well: fetched
+    // after the reduction they would put a second trip to the L2 on every row's critical path.
     float ss = 0.0f;
+    if (EARLY_WEIGHTS) {
+#pragma unroll
+      for (int i = 0; i < CACHE; ++i) wts[EARLY_WEIGHTS ? i : 0] = r2[min(tid + THREADS * i, nchunks - 1)];
+    }
 #pragma unroll
     for (int i = 0; i < CACHE; ++i) {
       const int c = tid + THREADS * i;
@@ -1773,7 +1779,7 @@ __global__ __launch_bounds__(THREADS) void fused_rowwise_quant_kernel(const uint
 #pragma unroll
       for (int e = 0; e < EPV; ++e) ss = __builtin_fmaf(f[e], f[e], ss);
     }
-    ss = block_reduce(ss, [](float a, float b) { return a + b; });
+    ss = block_reduce(0, ss, [](float a, float b) { return a + b; });
     rstd = 1.0f / sqrtf(ss / (float)K + eps);
   }
   // value of chunk c from its raw operands
@@ -1793,7 +1799,7 @@ __global__ __launch_bounds__(THREADS) void fused_rowwise_quant_kernel(const uint
     } else {
       V::unpack(__builtin_nontemporal_load(r1 + c), a);
     }
-    V::unpack(OP == kFusedRmsNorm ? r2[c] : __builtin_nontemporal_load(r2 + c), b);
+    V::unpack(EARLY_WEIGHTS ? wts[EARLY_WEIGHTS ? i : 0] : OP == kFusedRmsNorm ? r2[c] : __builtin_nontemporal_load(r2 + c), b);
     value(a, b, vals[i]);
 #pragma unroll
     for (int e = 0; e < EPV; ++e) amax = max_keep_nan(amax, fabsf(vals[i][e]));
@@ -1806,7 +1812,7 @@ __global__ __launch_bounds__(THREADS) void fused_rowwise_quant_kernel(const uint
 #pragma unroll
     for (int e = 0; e < EPV; ++e) amax = max_keep_nan(amax, fabsf(y[e]));
   }
-  amax = block_reduce(amax, [](float a, float b) { return max_keep_nan(a, b); });
+  amax = block_reduce(1, amax, [](float a, float b) { return max_keep_nan(a, b); });
 
   const float scale = row_scale<float>(amax);
   if (tid == 0) inv_scale[row] = 1.0f / scale;
