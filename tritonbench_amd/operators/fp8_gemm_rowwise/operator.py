@@ -171,6 +171,9 @@ class Operator(BenchmarkOperator):
     def _scaled_mm(self, xq, wq, x_scale, w_scale, bias) -> Callable:
         if not xq.is_cuda:
             raise NotImplementedError("torch._scaled_mm row-wise scaling needs a GPU")
+        if xq.shape[1] % 16 or wq.shape[0] % 16:
+            # the library refuses these at call time with a RuntimeError; the table shows "not supported" instead
+            raise NotImplementedError("torch._scaled_mm needs K and N divisible by 16")
         xs, ws = x_scale[:, None].contiguous(), w_scale[None, :].contiguous()
         return lambda: torch._scaled_mm(xq, wq.t(), scale_a=xs, scale_b=ws, bias=bias, out_dtype=torch.bfloat16)
 
