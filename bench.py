@@ -412,60 +412,91 @@ def main():
     if not args.no_extra:
         configs = {}
         cpu = not args.no_cpu_baseline
-        # C3: decode-sized, HBM-bound. Cold = rotate through operand sets larger than every cache.
-        cm, cn, ck = 16, 8192, 8192
-        cold_sets, cws = make_sets(cm, make_weights(cn, ck, 1.0, False, dev, 10), 1.0, dev)
-        cold = gemm_row(cm, cold_sets, cws, 200)
-        warm = gemm_row(cm, cold_sets[:1], cws, 200)
-        configs["c3_skinny_16x8192x8192"] = {"cold": cold, "cache_resident": warm}
-        if cpu:
-            configs["c3_skinny_16x8192x8192"]["cpu_baseline"] = cpu_baseline(cold_sets[0], "M=16, N=K=8192", budget_s=4.0)
-        del cold_sets
-        straffic, snote = measured_traffic("skinny")
-        # What one launch costs before any byte moves: the period of back-to-back launches of a kernel
-        # that touches 4 bytes, in the same kind of captured graph. It is part of every step above
-        # (10 % of the decode shape's), and no kernel of ours can remove it.
-        tiny = torch.zeros(1, device=dev)
-        floor_ms, _ = time_graph(lambda i: tiny.add_(1.0), 400)
-        line["launch_floor_us"] = floor_ms * 1e3
-        line["hbm_metric"] = {
-            "metric": "fp8_gemm_rowwise HBM GB/s at M=16,N=K=8192 (cold operands)",
-            "value": cold["gbps"], "unit": "GB/s", "us": cold["us"], "us_median": cold["us_median"],
-            "roofline": {"bound": "hbm", "achieved": cold["gbps"], "peak": PEAK_HBM_GBPS, "unit": "GB/s",
-                         "frac": cold["gbps"] / PEAK_HBM_GBPS, "traffic": straffic, **snote},
-            "frac_net_of_launch_floor": cold["gbps"] / PEAK_HBM_GBPS * cold["us"] / max(cold["us"] - floor_ms * 1e3, 1e-3),
-        }
-        # C5: ragged shapes with fused bias
-        for (rm, rn, rk) in [(1000, 3000, 4112), (4097, 7168, 2048)]:
-            rs, rws = make_sets(rm, make_weights(rn, rk, 1.0, True, dev, 2), 1.0, dev)
-            name = f"c5_ragged_bias_{rm}x{rn}x{rk}"
-            configs[name] = gemm_row(rm, rs, rws, 50)
+
+        def attempt(name, fn):
+            """One side workload. A failure is recorded in its place (and on stderr) and the
+            line, whose headline is already measured, is still printed."""
+            try:
+                configs[name] = fn()
+            except Exception as e:  # noqa: BLE001 - whatever it was, the record says so
+                configs[name] = {"error": f"{type(e).__name__}: {e}"}
+                print(f"bench.py: {name} failed: {type(e).__name__}: {e}", file=sys.stderr, flush=True)
+
+        def c3():
+            # C3: decode-sized, HBM-bound. Cold = rotate through operand sets larger than every cache.
+            cm, cn, ck = 16, 8192, 8192
+            cold_sets, cws = make_sets(cm, make_weights(cn, ck, 1.0, False, dev, 10), 1.0, dev)
+            cold = gemm_row(cm, cold_sets, cws, 200)
+            warm = gemm_row(cm, cold_sets[:1], cws, 200)
+            row = {"cold": cold, "cache_resident": warm}
             if cpu:
-                configs[name]["cpu_baseline"] = cpu_baseline(rs[0], f"{rm}x{rn}x{rk} + bias", budget_s=4.0, max_calls=3)
-            del rs
-        configs["c2_square_8192_graph"] = gemm_row(m, head_sets, head_ws, 20)
-        # C1: the reference's CPU-runnable plumbing case, here on the device with the host figure beside it
-        ps, pws = make_sets(128, make_weights(256, 512, 1.0, False, dev, 1), 1.0, dev)
-        configs["c1_plumbing_128x256x512"] = gemm_row(128, ps, pws, 200)
-        if cpu:
-            configs["c1_plumbing_128x256x512"]["cpu_baseline"] = cpu_baseline(ps[0], "128x256x512", budget_s=1.0)
+                row["cpu_baseline"] = cpu_baseline(cold_sets[0], "M=16, N=K=8192", budget_s=4.0)
+            del cold_sets
+            straffic, snote = measured_traffic("skinny")
+            # What one launch costs before any byte moves: the period of back-to-back launches of a kernel
+            # that touches 4 bytes, in the same kind of captured graph. It is part of every step above
+            # (10 % of the decode shape's), and no kernel of ours can remove it.
+            tiny = torch.zeros(1, device=dev)
+            floor_ms, _ = time_graph(lambda i: tiny.add_(1.0), 400)
+            line["launch_floor_us"] = floor_ms * 1e3
+            line["hbm_metric"] = {
+                "metric": "fp8_gemm_rowwise HBM GB/s at M=16,N=K=8192 (cold operands)",
+                "value": cold["gbps"], "unit": "GB/s", "us": cold["us"], "us_median": cold["us_median"],
+                "roofline": {"bound": "hbm", "achieved": cold["gbps"], "peak": PEAK_HBM_GBPS, "unit": "GB/s",
+                             "frac": cold["gbps"] / PEAK_HBM_GBPS, "traffic": straffic, **snote},
+                "frac_net_of_launch_floor": cold["gbps"] / PEAK_HBM_GBPS * cold["us"] / max(cold["us"] - floor_ms * 1e3, 1e-3),
+            }
+            return row
+
+        attempt("c3_skinny_16x8192x8192", c3)
+
+        def c5(rm, rn, rk):
+            # C5: ragged shapes with fused bias
+            rs, rws = make_sets(rm, make_weights(rn, rk, 1.0, True, dev, 2), 1.0, dev)
+            row = gemm_row(rm, rs, rws, 50)
+            if cpu:
+                row["cpu_baseline"] = cpu_baseline(rs[0], f"{rm}x{rn}x{rk} + bias", budget_s=4.0, max_calls=3)
+            return row
+
+        for (rm, rn, rk) in [(1000, 3000, 4112), (4097, 7168, 2048)]:
+            attempt(f"c5_ragged_bias_{rm}x{rn}x{rk}", lambda: c5(rm, rn, rk))
+        attempt("c2_square_8192_graph", lambda: gemm_row(m, head_sets, head_ws, 20))
+
+        def c1():
+            # C1: the reference's CPU-runnable plumbing case, here on the device with the host figure beside it
+            ps, pws = make_sets(128, make_weights(256, 512, 1.0, False, dev, 1), 1.0, dev)
+            row = gemm_row(128, ps, pws, 200)
+            if cpu:
+                row["cpu_baseline"] = cpu_baseline(ps[0], "128x256x512", budget_s=1.0)
+            return row
+
+        attempt("c1_plumbing_128x256x512", c1)
+
+        def c4(lm, ln, lk, weights):
+            ls, lws = make_sets(lm, weights, 0.02, dev)
+            return gemm_row(lm, ls, lws, 30 if lm < 1024 else 10)
+
         # C4: Llama-3-70B projections, sigma 0.02; the weight copies of an (N, K) pair serve its whole M sweep
         for (ln, lk) in LLAMA3_70B_NK:
-            weights = make_weights(ln, lk, 0.02, False, dev, copies_for(ln, lk))
+            try:
+                weights = make_weights(ln, lk, 0.02, False, dev, copies_for(ln, lk))
+            except Exception as e:  # noqa: BLE001 - the weights did not fit or could not be made: every row of the pair says so
+                for lm in LLAMA3_70B_M:
+                    configs[f"c4_llama70b_{lm}x{ln}x{lk}"] = {"error": f"{type(e).__name__}: {e}"}
+                print(f"bench.py: weights {ln}x{lk} failed: {type(e).__name__}: {e}", file=sys.stderr, flush=True)
+                continue
             for lm in LLAMA3_70B_M:
-                ls, lws = make_sets(lm, weights, 0.02, dev)
-                configs[f"c4_llama70b_{lm}x{ln}x{lk}"] = gemm_row(lm, ls, lws, 30 if lm < 1024 else 10)
-                del ls, lws
+                attempt(f"c4_llama70b_{lm}x{ln}x{lk}", lambda: c4(lm, ln, lk, weights))
             del weights
             torch.cuda.empty_cache()
-        configs["grouped_g4_8192x4096x4096"] = time_grouped(4, 8192, 4096, 4096, dev)
-        configs["grouped_g16_8192x8192x8192"] = time_grouped(16, 8192, 8192, 8192, dev, steps=20)
-        configs["blockwise_8192x8192x8192"] = time_blockwise(8192, 8192, 8192, dev)
-        configs["quantise_f32_8192x8192"] = time_quantiser(8192, 8192, torch.float32, dev)
-        configs["quantise_bf16_8192x8192"] = time_quantiser(8192, 8192, torch.bfloat16, dev)
-        configs["quantise_bf16_57344x8192"] = time_quantiser(57344, 8192, torch.bfloat16, dev, steps=20, copies=2)
-        configs["rmsnorm_quantise_bf16_8192x8192"] = time_fused_front_end("rmsnorm", 8192, 8192, dev)
-        configs["silu_mul_quantise_bf16_8192x8192"] = time_fused_front_end("silu_mul", 8192, 8192, dev)
+        attempt("grouped_g4_8192x4096x4096", lambda: time_grouped(4, 8192, 4096, 4096, dev))
+        attempt("grouped_g16_8192x8192x8192", lambda: time_grouped(16, 8192, 8192, 8192, dev, steps=20))
+        attempt("blockwise_8192x8192x8192", lambda: time_blockwise(8192, 8192, 8192, dev))
+        attempt("quantise_f32_8192x8192", lambda: time_quantiser(8192, 8192, torch.float32, dev))
+        attempt("quantise_bf16_8192x8192", lambda: time_quantiser(8192, 8192, torch.bfloat16, dev))
+        attempt("quantise_bf16_57344x8192", lambda: time_quantiser(57344, 8192, torch.bfloat16, dev, steps=20, copies=2))
+        attempt("rmsnorm_quantise_bf16_8192x8192", lambda: time_fused_front_end("rmsnorm", 8192, 8192, dev))
+        attempt("silu_mul_quantise_bf16_8192x8192", lambda: time_fused_front_end("silu_mul", 8192, 8192, dev))
         line["configs"] = configs
 
     if not args.no_cpu_baseline:
