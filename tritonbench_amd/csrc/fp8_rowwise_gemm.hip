@@ -15,12 +15,15 @@
 //   splitk_finalize_kernel   adds the fp32 partial sums of a split-K launch, applies scales/bias.
 //   gemm_skinny_kernel       M <= 64: every workgroup owns 16 rows of B and all of K, its waves
 //                            split K between them and reduce through LDS; B is streamed once.
+//   gemm_skinny_persistent_kernel  M <= 16 (M <= 32 at K = 4096): one 16-wave workgroup per CU keeps
+//                            its share of A in registers and walks 16-row tiles of B.
 //   quantize_rows_*_kernel   row-wise e4m3fn quantiser (amax, scale, convert), one row per workgroup.
+//   fused_rowwise_quant_kernel  RMSNorm or SiLU-mul of bf16 rows followed by the same quantiser, one pass.
 //
 // Operand roles inside the MFMA are swapped on purpose (rows of B feed the instruction's
 // "A" port, rows of A its "B" port) so each lane ends up holding 4 consecutive columns n of
-// one output row m (16 bytes of fp32 for the epilogue's LDS turn, 8 bytes of bf16 in the
-// skinny kernel's direct stores).
+// one output row m (8 bytes of 16-bit results for the epilogue's LDS turn and for the skinny
+// kernels' direct stores).
 
 #include <hip/hip_runtime.h>
 #include <stdint.h>
@@ -152,9 +155,10 @@ __device__ __forceinline__ void tile_coords(int t, int tiles_m, int tiles_n, int
 // operand reads (consecutive lanes = consecutive rows, same logical chunk) then spread over
 // all banks. With a load distance of 2 steps A has two stages,
 // B three (2*32 KB + 3*32 KB = all 160 KB of a 256x256 tile's LDS); the 256x128 tile runs at a
-// distance of 3 (3*32 KB + 4*16 KB). (A distance of 4 was
-// measured on the 128x128 tile with one workgroup per CU and bought under 10 %: that tile is
-// bound by LDS bandwidth - its 64x64 wave tiles read 128 B/clk of operands - not by latency.)
+// distance of 3 (3*32 KB + 4*16 KB). (Distances of 3 and 4 were measured on the 128x128 tile with one
+// workgroup per CU and bought under 10 %: that tile is bound by what the L2->L1->LDS path delivers
+// per CU, about 48 bytes per clock against the 64 its two workgroups ask for at the full MFMA
+// rate, not by the latency of a load.)
 // ------------------------------------------------------------------------------------
 constexpr int kStepK = 128;
 constexpr int kDefaultDist = 2;  // steps a load runs ahead of its use; A ring = DIST stages, B ring = DIST + 1
