@@ -102,3 +102,25 @@ def test_grouped_and_blockwise_argument_checks_need_no_gpu():
     assert blockwise(None, None, None, None, None, 64, 64, 32768 + 128, 40000, 40000, 64, None) == _lib.ENOTSUP
     assert "K <=" in _lib.last_error()
     assert blockwise(None, None, None, None, None, 64, 64, 256, 256, 256, 64, None) == _lib.EINVAL
+
+
+def test_leading_dimension_limits_are_checked_on_the_host():
+    """A tile's rows are addressed with 32-bit byte offsets: 256 rows of A or B and 256 rows of
+    16-bit output must stay below 2^31 bytes. The check comes before any device call, so host
+    buffers (never dereferenced) can stand in for the operands."""
+    lib = _lib.load()
+    buf = ctypes.create_string_buffer(4096 + 64)
+    base = (ctypes.addressof(buf) + 63) & ~63  # 64-byte aligned stand-in for every operand
+    m, n, k = 16, 16, 16
+    limit_ab = (2 ** 31 - 1) // 256  # largest lda/ldb that passes, rounded down to a multiple of 16 below
+    limit_c = (2 ** 31 - 1) // 512
+
+    def call(lda, ldb, ldc):
+        return lib.mi355x_fp8_rowwise_gemm(base, base, base, base, None, base, m, n, k, lda, ldb, ldc, None, 0, 0, None)
+
+    too_wide = (limit_ab // 16 + 1) * 16
+    assert call(too_wide, 16, 16) == _lib.ENOTSUP and "leading dimension too large" in _lib.last_error()
+    assert call(16, too_wide, 16) == _lib.ENOTSUP and "leading dimension too large" in _lib.last_error()
+    assert call(16, 16, limit_c + 1) == _lib.ENOTSUP and "leading dimension too large" in _lib.last_error()
+    # smaller than the row is a different complaint
+    assert call(8, 16, 16) == _lib.EINVAL and "smaller than the row" in _lib.last_error()
