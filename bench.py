@@ -194,6 +194,8 @@ def gemm_row(m, sets, workspace, steps):
 def timed_calls(call, steps, preheat_ms=30.0):
     """ms per call of call(i) over `steps` calls (HIP events on the launch stream), after untimed
     calls for `preheat_ms`."""
+    call(0)  # (the first call of a kernel loads its code object: not part of the preheat)
+    torch.cuda.synchronize()
     t0, i = time.perf_counter(), 0
     while (time.perf_counter() - t0) * 1e3 < preheat_ms:
         for _ in range(5):
@@ -330,6 +332,9 @@ def profile_kernel(which, dev):
     elif which == "quantise":
         fig = {"f32": time_quantiser(8192, 8192, torch.float32, dev, steps=20),
                "bf16": time_quantiser(8192, 8192, torch.bfloat16, dev, steps=20)}
+    elif which == "fused":
+        fig = {"rmsnorm": time_fused_front_end("rmsnorm", 8192, 8192, dev, steps=20),
+               "silu_mul": time_fused_front_end("silu_mul", 8192, 8192, dev, steps=20)}
     elif which == "grouped":
         fig = time_grouped(4, 8192, 4096, 4096, dev, steps=20)
     elif which == "decode128":
@@ -353,7 +358,7 @@ def main():
                     help="untimed launches before the warmup steps, until the device clock has settled")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-extra", action="store_true", help="headline workload only")
-    ap.add_argument("--profile-kernel", choices=["tiled", "skinny", "quantise", "grouped", "decode128", "ragged"],
+    ap.add_argument("--profile-kernel", choices=["tiled", "skinny", "quantise", "fused", "grouped", "decode128", "ragged"],
                     help="run only that kernel's workload a few times (for rocprofv3 counter passes) and print its figures")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
