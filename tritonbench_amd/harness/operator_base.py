@@ -266,6 +266,9 @@ class BenchmarkOperator(metaclass=_PostInit):
         self.device = tb_args.device
         metrics = getattr(tb_args, "metrics", None)
         self.required_metrics = list(dict.fromkeys(_csv_list(metrics))) if metrics else list(self.DEFAULT_METRICS)
+        if getattr(tb_args, "rocprof_pmc", None) and "rocprof" in self.required_metrics \
+                and "rocprof_counters" not in self.required_metrics:
+            self.required_metrics.append("rocprof_counters")  # the counters get a column of their own
         R.REGISTERED_X_VALS.setdefault(self.name, "x_val")
         precision = getattr(tb_args, "precision", "bypass")
         if precision == "bypass":
@@ -408,6 +411,12 @@ class BenchmarkOperator(metaclass=_PostInit):
                     rows = rocprof.profile_backend(self.name, fn_name, input_id, self.tb_args, self._raw_extra_args)
                     rec.extra_metrics["rocprof"] = rocprof.format_rows(rows)
                     rec.extra_metrics["rocprof_us"] = sum(r["us_per_call"] for r in rows)
+                    pmc = [c for c in (getattr(self.tb_args, "rocprof_pmc", None) or "").split(",") if c]
+                    if pmc:  # a run of its own: counters are never collected together with a trace
+                        per_kernel = rocprof.profile_backend_counters(
+                            self.name, fn_name, input_id, pmc, self.tb_args, self._raw_extra_args,
+                            kernels=[r["name"] for r in rows])
+                        rec.extra_metrics["rocprof_counters"] = rocprof.format_counters(per_kernel)
             if "gpu_peak_mem" in want and self.device == "cuda":
                 torch.cuda.reset_peak_memory_stats()
                 fn()

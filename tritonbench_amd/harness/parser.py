@@ -34,5 +34,8 @@ def get_parser() -> argparse.ArgumentParser:
     p.add_argument("--export", choices=["input", "output", "both"], default=None,
                    help="dump the inputs and/or every backend's output as .pt files")
     p.add_argument("--export-dir", default=None, help="existing directory for --export")
+    p.add_argument("--rocprof-pmc", default=None,
+                   help="with --metrics rocprof: hardware counters (comma separated, one rocprofv3 pass) collected "
+                        "in a second child run and shown per kernel")
     p.add_argument("--list-backends", action="store_true")
     return p

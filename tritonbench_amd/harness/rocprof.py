@@ -244,6 +244,27 @@ def profile_backend(op_name: str, fn_name: str, input_id: int, tb_args=None, ext
     return window_stats(parse_kernel_trace(_find(where, "_kernel_trace.csv")))
 
 
+def profile_backend_counters(op_name: str, fn_name: str, input_id: int, counters: Sequence[str], tb_args=None,
+                             extra_args=None, kernels: Optional[Sequence[str]] = None,
+                             out_dir: Optional[str] = None) -> Dict[str, Dict[str, float]]:
+    """One counter pass over the same child: {short kernel name: {counter: mean per dispatch}} for the
+    kernels whose full names are in `kernels` (all of the child's kernels when None). The means are
+    over every dispatch of a kernel in the child, its warm-up calls included."""
+    check_pmc_fits(counters)
+    child = child_argv(op_name, fn_name, input_id, tb_args, extra_args)
+    where = run_profiler(child, pmc=list(counters), out_dir=out_dir)
+    table = parse_counters(_find(where, "_counter_collection.csv"))
+    keep = None if kernels is None else set(kernels)
+    return {short_kernel_name(name): {c: v["mean"] for c, v in per.items()}
+            for name, per in table.items() if keep is None or name in keep}
+
+
+def format_counters(per_kernel: Dict[str, Dict[str, float]]) -> str:
+    """One table cell: `kernel: COUNTER=mean, ...; ...`."""
+    return "; ".join(f"{k}: " + ", ".join(f"{c}={v:.6g}" for c, v in sorted(per.items()))
+                     for k, per in per_kernel.items())
+
+
 # ---- traffic summary for bench.py -----------------------------------------------------------
 
 def traffic_summary(fetch_csv: str, write_csv: str, kernel: str, copy_kernel: str, copy_read_bytes: int,
