@@ -1,6 +1,6 @@
 """Benchmark of the row-wise FP8 GEMM hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu-baseline] [--no-extra]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu-baseline] [--no-extra] [--vendor]
 
 One step = one pass of the hot path (one mi355x_fp8_rowwise_gemm call through the C ABI) over
 the headline workload M=N=K=8192 with operands resident in HBM. Prints ONE JSON line: the
@@ -185,10 +185,35 @@ def figures(m, n, k, bias, ms, ms_median=None):
     return row
 
 
+VENDOR = False  # --vendor: time torch._scaled_mm (hipBLASLt's row-wise FP8 GEMM) on the same operand sets
+
+
+def vendor_us(sets, steps):
+    """Microseconds per call of torch._scaled_mm with row-wise scales on the same rotated operand
+    sets, timed like our own rows (captured graph, best replay); None where the library refuses
+    the shape. The scale views are made once, outside the timed calls."""
+    prepared = [(xq, wq.t(), xs[:, None].contiguous(), ws[None, :].contiguous(), b) for (xq, wq, xs, ws, b, _) in sets]
+
+    def call(i):
+        a, bt, sa, sb, bias = prepared[i % len(prepared)]
+        torch._scaled_mm(a, bt, scale_a=sa, scale_b=sb, bias=bias, out_dtype=torch.bfloat16)
+
+    try:
+        best, _ = time_graph(call, steps)
+    except Exception as e:  # noqa: BLE001 - e.g. N or K not a multiple of 16
+        print(f"bench.py: torch._scaled_mm refused {tuple(sets[0][0].shape)} x {tuple(sets[0][1].shape)}: {e}",
+              file=sys.stderr, flush=True)
+        return None
+    return best * 1e3
+
+
 def gemm_row(m, sets, workspace, steps):
     xq, wq, _, _, b, _ = sets[0]
     best, med = time_graph(lambda i: launch(sets[i % len(sets)], workspace), steps)
-    return figures(m, wq.shape[0], wq.shape[1], b is not None, best, med)
+    row = figures(m, wq.shape[0], wq.shape[1], b is not None, best, med)
+    if VENDOR:
+        row["hipblaslt_us"] = vendor_us(sets, steps)
+    return row
 
 
 def timed_calls(call, steps, preheat_ms=30.0):
@@ -358,9 +383,13 @@ def main():
                     help="untimed launches before the warmup steps, until the device clock has settled")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-extra", action="store_true", help="headline workload only")
+    ap.add_argument("--vendor", action="store_true",
+                    help="also time torch._scaled_mm (hipBLASLt, row-wise scales) on every GEMM row's operands")
     ap.add_argument("--profile-kernel", choices=["tiled", "skinny", "quantise", "fused", "grouped", "decode128", "ragged"],
                     help="run only that kernel's workload a few times (for rocprofv3 counter passes) and print its figures")
     args = ap.parse_args()
+    global VENDOR
+    VENDOR = args.vendor
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py measures one GPU: this hot path is a single-device kernel and nothing here "
               "uses a second GPU; run with --gpus 1", file=sys.stderr)
