@@ -68,6 +68,8 @@ def test_automatic_choice_is_close_to_the_best_alternative(gpu_device, m, n, k, 
     if m <= 64:
         alternatives["skinny"] = _lib.VARIANT_SKINNY
         alternatives["skinny, one tile per workgroup"] = _lib.VARIANT_SKINNY | _lib.SKINNY_ONE_TILE
+        if k % 512 == 0:
+            alternatives["skinny, narrow tiles"] = _lib.VARIANT_SKINNY | _lib.SKINNY_NARROW
     # two rounds over all candidates, the automatic choice first and last: whatever is timed first
     # runs on a colder clock
     # (a third round only if the bound does not hold after two: one noisy replay must not fail the suite)

@@ -333,9 +333,12 @@ def test_dispatch_is_pinned(gpu_device):
     assert ops.select_variant(16, 8192, 8192) == _lib.VARIANT_SKINNY
     assert ops.select_variant(32, 2048, 2048) == _lib.VARIANT_SKINNY
     assert ops.select_variant(8192, 8192, 8192) == _lib.VARIANT_TILED
-    # three or four 16-row blocks of A, or two with a long weight panel: split-K tiles that
-    # fetch B with the streaming policy win
-    assert ops.select_variant(64, 8192, 8192) == _lib.VARIANT_TILED
+    # up to 64 rows against a panel that gives every CU at most one 32-column tile: the M <= 64
+    # family's narrow-tile form
+    assert ops.select_variant(64, 8192, 8192) == _lib.VARIANT_SKINNY
+    assert ops.select_variant(32, 8192, 28672) == _lib.VARIANT_SKINNY
+    # three or four 16-row blocks of A against more tiles than CUs, or two with a long weight
+    # panel: split-K tiles that fetch B with the streaming policy win
     assert ops.select_variant(48, 10240, 8192) == _lib.VARIANT_TILED
     assert ops.select_variant(64, 57344, 8192) == _lib.VARIANT_TILED
     assert ops.select_variant(32, 57344, 8192) == _lib.VARIANT_TILED

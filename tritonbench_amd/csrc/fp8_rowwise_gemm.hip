@@ -17,6 +17,8 @@
 //                            split K between them and reduce through LDS; B is streamed once.
 //   gemm_skinny_persistent_kernel  M <= 16 (M <= 32 at K = 4096): one 16-wave workgroup per CU keeps
 //                            its share of A in registers and walks 16-row tiles of B.
+//   gemm_narrow_kernel       M <= 64, K in 512-byte steps, at most one 32-column tile per CU: a workgroup
+//                            owns all of K (no split, no second launch); separate waves fetch A and B.
 //   quantize_rows_*_kernel   row-wise e4m3fn quantiser (amax, scale, convert), one row per workgroup.
 //   fused_rowwise_quant_kernel  RMSNorm or SiLU-mul of bf16 rows followed by the same quantiser, one pass.
 //
@@ -1489,6 +1491,195 @@ __global__ __launch_bounds__(kPersistWaves * 64) void gemm_skinny_persistent_ker
 }
 
 // ------------------------------------------------------------------------------------
+// Narrow-tile kernel for M <= 32*MB (MB = 1, 2), K a multiple of 512: one workgroup per 32
+// columns of C owns all of K, so there are no partial sums and no second launch. It is the
+// form for panels that give every CU at most one such tile (N <= 8192) when A has more rows
+// than the persistent kernel above keeps in registers.
+//
+// Eight waves. A K step is 512 bytes: wave w of the first four fetches and multiplies the
+// step's w-th 128-byte slab of A (rows of A are L2 hits: a short queue, DA steps ahead), wave
+// 4+w fetches the same slab of the tile's 32 rows of B (from HBM, kNarrowBDist steps ahead).
+// Loads return to a wave in order: with A and B in one queue every A line would wait behind
+// the B lines in front of it and see HBM's latency. Both go straight into LDS stages laid out
+// as [slab][row][128 bytes] with the tiled kernel's chunk swizzle; one barrier per step. The
+// four partial 32x32 (x MB) results meet in LDS at the end; wave w finishes columns 8w..8w+7
+// of every 32-row block.
+// Workgroup g starts its walk over K at step 5g mod steps and wraps around: with a power-of-two
+// row pitch the rows in flight at one moment would otherwise agree in their low address bits
+// and crowd a few memory channels (measured, M=32, N=K=8192, K loop only: 19.8 -> 13.4 us).
+// ------------------------------------------------------------------------------------
+constexpr int kNarrowKS = 512;
+constexpr int kNarrowBDist = 5;
+constexpr int narrow_a_dist(int MB) { return MB == 1 ? 2 : 1; }
+constexpr size_t narrow_lds_bytes(int MB) {
+  return (size_t)(narrow_a_dist(MB) + 1) * MB * 32 * kNarrowKS + (size_t)(kNarrowBDist + 1) * 32 * kNarrowKS;
+}
+static_assert(narrow_lds_bytes(2) <= 160 * 1024, "stage rings must fit the LDS");
+
+// waits until at most VM of this wave's global loads are outstanding (LDS operations are not waited for)
+template <int VM>
+__device__ __forceinline__ void wait_loads() {
+  constexpr int imm = (VM & 15) | ((VM >> 4) << 14) | (7 << 4) | (15 << 8);
+  __builtin_amdgcn_s_waitcnt(imm);
+}
+
+template <int MB>
+__global__ __launch_bounds__(512) void gemm_narrow_kernel(GemmParams p) {
+  constexpr int BM = 32 * MB, KS = kNarrowKS, DA = narrow_a_dist(MB), DB = kNarrowBDist;
+  constexpr int RA = DA + 1, RB = DB + 1;
+  constexpr int STA = BM * KS, STB = 32 * KS;  // bytes per stage
+  constexpr int LA = BM / 8, LB = 4;           // wave-wide loads per wave and step (8 rows x 128 bytes each)
+  static_assert((DA - 1) * LA < 64 && (DB - 1) * LB < 64, "outstanding-load counts must fit the wait instruction");
+  extern __shared__ __attribute__((aligned(1024))) uint8_t lds[];
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int n0 = blockIdx.x * 32;
+  const int ksteps = p.K / KS;
+  const int rot = (int)((blockIdx.x * 5u) % (unsigned)ksteps);
+  // a lane's 16 bytes of an 8-row group: row lane/8; LDS position lane%8 holds logical chunk
+  // position ^ key(row), key = (row >> 1) & 7: for the even groups of a slab that is ld_row >> 1, for
+  // the odd ones 4 more, which flips bit 6 of the byte offset
+  const int ld_row = lane >> 3, ld_pc = lane & 7;
+  const uint32_t chunk_even = (uint32_t)((ld_pc ^ (ld_row >> 1)) * kChunk);
+  auto step_of = [&](int s) { const int t = s + rot; return t >= ksteps ? t - ksteps : t; };
+
+  if (wave < 4) {
+    // ---- compute wave: slab `wave` of every step
+    const __amdgpu_buffer_rsrc_t ra = __builtin_amdgcn_make_buffer_rsrc(
+        const_cast<uint8_t*>(p.a), 0, (int)((uint32_t)min(p.M, BM) * (uint32_t)p.lda), 0x00020000);
+    const uint32_t a_even = (uint32_t)ld_row * (uint32_t)p.lda + chunk_even;
+    const uint32_t a_odd = (uint32_t)ld_row * (uint32_t)p.lda + (chunk_even ^ 64u);
+    auto issue_a = [&](int s) {
+      if (s >= ksteps) return;
+      uint8_t* dst = lds + (s % RA) * STA + wave * (BM * kStepK);
+      const uint32_t koff = (uint32_t)step_of(s) * KS + (uint32_t)wave * kStepK;
+#pragma unroll
+      for (int g = 0; g < LA; ++g)
+        load_chunk_to_lds<false>(ra, dst + g * 1024, (g & 1) ? a_odd : a_even, (uint32_t)(g * 8) * (uint32_t)p.lda + koff);
+    };
+    // this lane's scales and bias, asked for before the loop: row l32 of every block, columns
+    // n0 + 8*wave + 4*half .. +3 (indices clamped; what lies past an edge is never stored)
+    const int l32 = lane & 31, half = lane >> 5;
+    const int nq = n0 + 8 * wave + 4 * half;
+    float sa[MB], sb[4], bias_f[4];
+#pragma unroll
+    for (int i = 0; i < MB; ++i) sa[i] = p.a_scale[min(i * 32 + l32, p.M - 1)];
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      const int ne = min(nq + e, p.N - 1);
+      sb[e] = p.b_scale[ne];
+      bias_f[e] = p.bias ? bf16_to_f32(p.bias[ne]) : 0.0f;
+    }
+#pragma unroll
+    for (int s = 0; s < DA; ++s) issue_a(s);
+    if (ksteps > DA) wait_loads<(DA - 1) * LA>(); else wait_loads<0>();
+    __builtin_amdgcn_s_barrier();
+
+    v16f acc[MB];
+    const v16f zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int i = 0; i < MB; ++i) acc[i] = zero;
+    // fragment of K half sh (64 bytes) of this wave's slab: logical chunks 4*half + 2*sh + {0, 1} of row l32
+    int rd[2][2];
+#pragma unroll
+    for (int sh = 0; sh < 2; ++sh)
+#pragma unroll
+      for (int j = 0; j < 2; ++j) rd[sh][j] = l32 * kStepK + (((4 * half + 2 * sh + j) ^ swz128(l32)) * kChunk);
+
+    for (int s = 0; s < ksteps; ++s) {
+      issue_a(s + DA);
+      const uint8_t* sa_rows = lds + (s % RA) * STA + wave * (BM * kStepK);
+      const uint8_t* sb_rows = lds + RA * STA + (s % RB) * STB + wave * (32 * kStepK);
+      v4i fb[2][2], fa[MB][2][2];
+#pragma unroll
+      for (int sh = 0; sh < 2; ++sh) {
+#pragma unroll
+        for (int j = 0; j < 2; ++j) fb[sh][j] = *(const v4i*)(sb_rows + rd[sh][j]);
+#pragma unroll
+        for (int i = 0; i < MB; ++i)
+#pragma unroll
+          for (int j = 0; j < 2; ++j) fa[i][sh][j] = *(const v4i*)(sa_rows + i * 32 * kStepK + rd[sh][j]);
+      }
+#pragma unroll
+      for (int sh = 0; sh < 2; ++sh) {
+        const v8i vb = (v8i){fb[sh][0][0], fb[sh][0][1], fb[sh][0][2], fb[sh][0][3],
+                             fb[sh][1][0], fb[sh][1][1], fb[sh][1][2], fb[sh][1][3]};
+#pragma unroll
+        for (int i = 0; i < MB; ++i) {
+          const v8i va = (v8i){fa[i][sh][0][0], fa[i][sh][0][1], fa[i][sh][0][2], fa[i][sh][0][3],
+                               fa[i][sh][1][0], fa[i][sh][1][1], fa[i][sh][1][2], fa[i][sh][1][3]};
+          acc[i] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(vb, va, acc[i], 0, 0, 0, 0, 0, 0);
+        }
+      }
+      // own loads of A(s+1) have landed (the younger A(s+2) .. A(s+DA) may be in flight); past the barrier
+      // everyone's have, B's included, and every wave is done reading this step's stages
+      if (s + DA < ksteps) wait_loads<(DA - 1) * LA>(); else wait_loads<0>();
+      __builtin_amdgcn_s_barrier();
+    }
+
+    // ---- the four waves' partial results meet in LDS (the stages are free: last barrier passed)
+    v4f* area = (v4f*)lds;  // [wave][block][q][lane]
+#pragma unroll
+    for (int i = 0; i < MB; ++i)
+#pragma unroll
+      for (int q = 0; q < 4; ++q)
+        area[((wave * MB + i) * 4 + q) * 64 + lane] = (v4f){acc[i][4 * q], acc[i][4 * q + 1], acc[i][4 * q + 2], acc[i][4 * q + 3]};
+    __syncthreads();
+    const bool vec = ((p.ldc & 3) == 0) && ((reinterpret_cast<uintptr_t>(p.c) & 7) == 0);
+#pragma unroll
+    for (int i = 0; i < MB; ++i) {
+      v4f sum = area[((0 * MB + i) * 4 + wave) * 64 + lane];
+#pragma unroll
+      for (int w = 1; w < 4; ++w) sum += area[((w * MB + i) * 4 + wave) * 64 + lane];
+      const int m = i * 32 + l32;
+      if (m < p.M && nq < p.N) {
+        float r[4];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          const float t = sum[e] * sa[i];
+          r[e] = p.bias ? __builtin_fmaf(t, sb[e], bias_f[e]) : t * sb[e];
+        }
+        const uint32_t lo = pack_out_x2(r[0], r[1], p.out_f16), hi = pack_out_x2(r[2], r[3], p.out_f16);
+        uint16_t* dst = p.c + (size_t)m * p.ldc + nq;
+        if (vec && nq + 3 < p.N) {
+          *(v2u*)dst = (v2u){lo, hi};
+        } else {
+          dst[0] = (uint16_t)lo;
+          if (nq + 1 < p.N) dst[1] = (uint16_t)(lo >> 16);
+          if (nq + 2 < p.N) dst[2] = (uint16_t)hi;
+          if (nq + 3 < p.N) dst[3] = (uint16_t)(hi >> 16);
+        }
+      }
+    }
+  } else {
+    // ---- loader wave for B: slab `wave - 4` of every step, 8 rows per load
+    const int w = wave - 4;
+    const __amdgpu_buffer_rsrc_t rb = __builtin_amdgcn_make_buffer_rsrc(
+        const_cast<uint8_t*>(p.b) + (size_t)n0 * p.ldb, 0, (int)((uint32_t)min(p.N - n0, 32) * (uint32_t)p.ldb), 0x00020000);
+    const uint32_t b_even = (uint32_t)ld_row * (uint32_t)p.ldb + chunk_even;
+    const uint32_t b_odd = (uint32_t)ld_row * (uint32_t)p.ldb + (chunk_even ^ 64u);
+    auto issue_b = [&](int s) {
+      if (s >= ksteps) return;
+      uint8_t* dst = lds + RA * STA + (s % RB) * STB + w * (32 * kStepK);
+      const uint32_t koff = (uint32_t)step_of(s) * KS + (uint32_t)w * kStepK;
+#pragma unroll
+      for (int g = 0; g < LB; ++g)
+        load_chunk_to_lds<true>(rb, dst + g * 1024, (g & 1) ? b_odd : b_even, (uint32_t)(g * 8) * (uint32_t)p.ldb + koff);
+    };
+#pragma unroll
+    for (int s = 0; s < DB; ++s) issue_b(s);
+    if (ksteps > DB) wait_loads<(DB - 1) * LB>(); else wait_loads<0>();
+    __builtin_amdgcn_s_barrier();
+    for (int s = 0; s < ksteps; ++s) {
+      issue_b(s + DB);
+      if (s + DB < ksteps) wait_loads<(DB - 1) * LB>(); else wait_loads<0>();
+      __builtin_amdgcn_s_barrier();
+    }
+    __syncthreads();  // the compute waves' hand-over of their partial results
+  }
+}
+
+// ------------------------------------------------------------------------------------
 // Row-wise quantiser: one workgroup per row, two passes over the row (amax, then scale
 // and convert). e4m3fn encoding is done with integer arithmetic so the rounding
 // (nearest, ties to even, subnormals below 2^-6) does not depend on conversion hardware.
@@ -1925,7 +2116,19 @@ constexpr TileConfig kTileConfigs[kNumTileConfigs] = {
 // four blocks the register budget leaves one workgroup per CU, and a last round of workgroups
 // that fills only part of the CUs streams at that fraction of the rate.
 inline bool persistent_skinny_fits(int64_t M, int64_t N, int64_t K);
-inline float skinny_cost_us(int64_t M, int64_t N, int64_t K) {
+// The narrow-tile kernel: M <= 64, K in whole 512-byte steps. Its cost is one round of workgroups per
+// 256 tiles (measured at N = 8192, cold: 9.8 / 14.3 / 43.0 us for K = 4096 / 8192 / 28672 with up to
+// 32 rows of A, 17.1-17.9 / 49.9 us for K = 8192 / 28672 with up to 64).
+inline bool narrow_fits(int64_t M, int64_t N, int64_t K) {
+  (void)N;
+  return M <= 64 && K % 512 == 0;
+}
+inline float narrow_cost_us(int64_t M, int64_t N, int64_t K) {
+  const long tiles = (N + 31) / 32;
+  const long rounds = (tiles + kNumCu - 1) / kNumCu;
+  return (float)rounds * (M <= 32 ? 3.5f + (float)K / 1024.0f * 1.38f : 4.5f + (float)K / 1024.0f * 1.62f);
+}
+inline float skinny_streaming_cost_us(int64_t M, int64_t N, int64_t K) {
   // the persistent form (measured: 12.7 us at N=K=8192, 71 us at N=57344)
   // (two blocks of A, K = 4096: 9.9 us at N=8192)
   if (persistent_skinny_fits(M, N, K)) return 3.0f + (float)N * (float)K / (M <= 16 ? 6.9e6f : 4.9e6f);
@@ -1941,6 +2144,13 @@ inline float skinny_cost_us(int64_t M, int64_t N, int64_t K) {
     r *= (float)wgs / (float)(rounds * kNumCu);
   }
   return 5.0f + (float)N * (float)K / r;
+}
+// the cheapest member of the M <= 64 family: streaming (persistent or one tile per workgroup) or narrow tiles
+inline bool narrow_preferred(int64_t M, int64_t N, int64_t K) {
+  return narrow_fits(M, N, K) && narrow_cost_us(M, N, K) < skinny_streaming_cost_us(M, N, K);
+}
+inline float skinny_cost_us(int64_t M, int64_t N, int64_t K) {
+  return narrow_preferred(M, N, K) ? narrow_cost_us(M, N, K) : skinny_streaming_cost_us(M, N, K);
 }
 constexpr int kMaxSplits = 16;
 // Tile rows up to which a launch fetches B with the streaming policy (see gemm_tiled_kernel).
@@ -2184,6 +2394,19 @@ int launch_skinny_persistent_steps(const GemmParams& p, hipStream_t s) {
   }
 }
 
+template <int MB>
+int launch_narrow(const GemmParams& p, hipStream_t stream) {
+  constexpr size_t lds_bytes = narrow_lds_bytes(MB);
+  auto kern = gemm_narrow_kernel<MB>;
+  static bool attr_done[kMaxDevices] = {};
+  if (const int st = raise_lds_limit((const void*)kern, lds_bytes, attr_done)) return st;
+  const unsigned grid = (unsigned)((p.N + 31) / 32);
+  hipLaunchKernelGGL(kern, dim3(grid), dim3(512), lds_bytes, stream, p);
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess) return fail(MI355X_FP8_ELAUNCH, "narrow-tile kernel launch: %s", hipGetErrorString(e));
+  return MI355X_FP8_OK;
+}
+
 }  // namespace
 
 extern "C" {
@@ -2303,6 +2526,14 @@ int mi355x_fp8_rowwise_gemm_ex(const void* a, const void* b, const float* a_scal
       // 16-row blocks of A | B tiles per wave | steps in flight per wave (sized to 128 VGPRs) | waves.
       // (Measured alternatives at M = 16: two B tiles per wave with 4, 6 or 8 steps in flight 17.8-19.9 us,
       // four waves 14.7-15.0 us, six steps in flight 16.4 us, against 14.4 us for this one.)
+      if (plan_bits & MI355X_FP8_SKINNY_NARROW) {
+        if (!narrow_fits(M, N, K))
+          return fail(MI355X_FP8_ENOTSUP, "the narrow-tile kernel takes M <= 64 and K in multiples of 512 (got M=%lld, K=%lld)",
+                      (long long)M, (long long)K);
+        return M <= 32 ? launch_narrow<1>(p, s) : launch_narrow<2>(p, s);
+      }
+      if (!(plan_bits & MI355X_FP8_SKINNY_ONE_TILE) && narrow_preferred(M, N, K))
+        return M <= 32 ? launch_narrow<1>(p, s) : launch_narrow<2>(p, s);
       if (persistent_skinny_fits(M, N, K) && !(plan_bits & MI355X_FP8_SKINNY_ONE_TILE)) {
         // 16-byte loads of b_scale, 8-byte loads of bias and 8-byte stores of C when everything is aligned for them
         const bool vec = (reinterpret_cast<uintptr_t>(b_scale) & 15) == 0 && (reinterpret_cast<uintptr_t>(bias) & 7) == 0 &&
