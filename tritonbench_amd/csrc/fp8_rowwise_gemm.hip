@@ -1504,17 +1504,19 @@ __global__ __launch_bounds__(kPersistWaves * 64) void gemm_skinny_persistent_ker
 // as [slab][row][128 bytes] with the tiled kernel's chunk swizzle; one barrier per step. The
 // four partial 32x32 (x MB) results meet in LDS at the end; wave w finishes columns 8w..8w+7
 // of every 32-row block.
+// SHARED halves the ring depths so that two workgroups fit a CU: for panels of one to two tiles per CU.
 // Workgroup g starts its walk over K at step 5g mod steps and wraps around: with a power-of-two
 // row pitch the rows in flight at one moment would otherwise agree in their low address bits
 // and crowd a few memory channels (measured, M=32, N=K=8192, K loop only: 19.8 -> 13.4 us).
 // ------------------------------------------------------------------------------------
 constexpr int kNarrowKS = 512;
-constexpr int kNarrowBDist = 5;
-constexpr int narrow_a_dist(int MB) { return MB == 1 ? 2 : 1; }
-constexpr size_t narrow_lds_bytes(int MB) {
-  return (size_t)(narrow_a_dist(MB) + 1) * MB * 32 * kNarrowKS + (size_t)(kNarrowBDist + 1) * 32 * kNarrowKS;
+// SHARED: rings half as deep, so that two workgroups fit a CU (for tile counts between one and two per CU)
+constexpr int narrow_b_dist(bool shared) { return shared ? 2 : 5; }
+constexpr int narrow_a_dist(int MB, bool shared) { return MB == 1 && !shared ? 2 : 1; }
+constexpr size_t narrow_lds_bytes(int MB, bool shared) {
+  return (size_t)(narrow_a_dist(MB, shared) + 1) * MB * 32 * kNarrowKS + (size_t)(narrow_b_dist(shared) + 1) * 32 * kNarrowKS;
 }
-static_assert(narrow_lds_bytes(2) <= 160 * 1024, "stage rings must fit the LDS");
+static_assert(narrow_lds_bytes(2, false) <= 160 * 1024 && narrow_lds_bytes(1, true) <= 80 * 1024, "stage rings must fit the LDS");
 
 // waits until at most VM of this wave's global loads are outstanding (LDS operations are not waited for)
 template <int VM>
@@ -1523,9 +1525,9 @@ __device__ __forceinline__ void wait_loads() {
   __builtin_amdgcn_s_waitcnt(imm);
 }
 
-template <int MB>
+template <int MB, bool SHARED>
 __global__ __launch_bounds__(512) void gemm_narrow_kernel(GemmParams p) {
-  constexpr int BM = 32 * MB, KS = kNarrowKS, DA = narrow_a_dist(MB), DB = kNarrowBDist;
+  constexpr int BM = 32 * MB, KS = kNarrowKS, DA = narrow_a_dist(MB, SHARED), DB = narrow_b_dist(SHARED);
   constexpr int RA = DA + 1, RB = DB + 1;
   constexpr int STA = BM * KS, STB = 32 * KS;  // bytes per stage
   constexpr int LA = BM / 8, LB = 4;           // wave-wide loads per wave and step (8 rows x 128 bytes each)
@@ -2123,7 +2125,15 @@ inline bool narrow_fits(int64_t M, int64_t N, int64_t K) {
   (void)N;
   return M <= 64 && K % 512 == 0;
 }
+// Between one and two tiles per CU, with one block of A: rings half as deep, two workgroups per CU, all
+// tiles resident at once instead of two rounds (measured at K = 8192, M = 32: 22.3 / 23.9 / 24.1 us for
+// N = 10240 / 12288 / 16384; 13.4 us at N = 10240, K = 4096).
+inline bool narrow_shares_cus(int64_t M, int64_t N) {
+  const long tiles = (N + 31) / 32;
+  return M <= 32 && tiles > kNumCu && tiles <= 2 * kNumCu;
+}
 inline float narrow_cost_us(int64_t M, int64_t N, int64_t K) {
+  if (narrow_shares_cus(M, N)) return 4.5f + (float)K / 1024.0f * 2.4f;
   const long tiles = (N + 31) / 32;
   const long rounds = (tiles + kNumCu - 1) / kNumCu;
   return (float)rounds * (M <= 32 ? 3.5f + (float)K / 1024.0f * 1.38f : 4.5f + (float)K / 1024.0f * 1.62f);
@@ -2394,10 +2404,10 @@ int launch_skinny_persistent_steps(const GemmParams& p, hipStream_t s) {
   }
 }
 
-template <int MB>
+template <int MB, bool SHARED = false>
 int launch_narrow(const GemmParams& p, hipStream_t stream) {
-  constexpr size_t lds_bytes = narrow_lds_bytes(MB);
-  auto kern = gemm_narrow_kernel<MB>;
+  constexpr size_t lds_bytes = narrow_lds_bytes(MB, SHARED);
+  auto kern = gemm_narrow_kernel<MB, SHARED>;
   static bool attr_done[kMaxDevices] = {};
   if (const int st = raise_lds_limit((const void*)kern, lds_bytes, attr_done)) return st;
   const unsigned grid = (unsigned)((p.N + 31) / 32);
@@ -2530,10 +2540,13 @@ int mi355x_fp8_rowwise_gemm_ex(const void* a, const void* b, const float* a_scal
         if (!narrow_fits(M, N, K))
           return fail(MI355X_FP8_ENOTSUP, "the narrow-tile kernel takes M <= 64 and K in multiples of 512 (got M=%lld, K=%lld)",
                       (long long)M, (long long)K);
+        if (narrow_shares_cus(M, N)) return launch_narrow<1, true>(p, s);
         return M <= 32 ? launch_narrow<1>(p, s) : launch_narrow<2>(p, s);
       }
-      if (!(plan_bits & MI355X_FP8_SKINNY_ONE_TILE) && narrow_preferred(M, N, K))
+      if (!(plan_bits & MI355X_FP8_SKINNY_ONE_TILE) && narrow_preferred(M, N, K)) {
+        if (narrow_shares_cus(M, N)) return launch_narrow<1, true>(p, s);
         return M <= 32 ? launch_narrow<1>(p, s) : launch_narrow<2>(p, s);
+      }
       if (persistent_skinny_fits(M, N, K) && !(plan_bits & MI355X_FP8_SKINNY_ONE_TILE)) {
         // 16-byte loads of b_scale, 8-byte loads of bias and 8-byte stores of C when everything is aligned for them
         const bool vec = (reinterpret_cast<uintptr_t>(b_scale) & 15) == 0 && (reinterpret_cast<uintptr_t>(bias) & 7) == 0 &&
