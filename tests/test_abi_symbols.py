@@ -44,7 +44,7 @@ def test_host_side_argument_checks_need_no_gpu():
     assert lib.mi355x_fp8_rowwise_select_variant(8192, 8192, 8192) == _lib.VARIANT_TILED
     assert lib.mi355x_fp8_rowwise_select_variant(32, 2048, 2048) == _lib.VARIANT_SKINNY
     assert lib.mi355x_fp8_rowwise_select_variant(64, 8192, 8192) == _lib.VARIANT_SKINNY  # (its narrow-tile form)
-    assert lib.mi355x_fp8_rowwise_select_variant(64, 10240, 8192) == _lib.VARIANT_TILED
+    assert lib.mi355x_fp8_rowwise_select_variant(64, 28672, 8192) == _lib.VARIANT_TILED
     assert lib.mi355x_fp8_rowwise_select_variant(64, 57344, 8192) == _lib.VARIANT_TILED
     assert lib.mi355x_fp8_rowwise_select_variant(0, 8, 16) == _lib.EINVAL
     assert lib.mi355x_fp8_rowwise_select_variant(8, 8, 24) == _lib.ENOTSUP

@@ -56,8 +56,9 @@ SHAPES = [
     (20, 999, 2048, True), (32, 8192, 4096, False), (31, 4100, 3072, True), (24, 8224, 2048, False),
     (33, 64, 512, True), (64, 8192, 2048, False), (50, 1000, 4096, True), (64, 33, 2560, False),
     (48, 2056, 8192, True), (32, 1024, 28672, False), (64, 520, 8192, True),
-    # between one and two tiles per CU with one block of A: the form with two workgroups per CU
+    # between one and two 32-column tiles per CU: 64-column tiles, with one and two blocks of A
     (32, 16384, 2048, True), (20, 10250, 1024, False), (7, 12288, 512, True), (32, 8224, 4096, False),
+    (64, 16384, 1024, False), (40, 9001, 2560, True), (64, 8250, 512, True),
 ]
 
 

@@ -337,9 +337,10 @@ def test_dispatch_is_pinned(gpu_device):
     # family's narrow-tile form
     assert ops.select_variant(64, 8192, 8192) == _lib.VARIANT_SKINNY
     assert ops.select_variant(32, 8192, 28672) == _lib.VARIANT_SKINNY
-    # three or four 16-row blocks of A against more tiles than CUs, or two with a long weight
-    # panel: split-K tiles that fetch B with the streaming policy win
-    assert ops.select_variant(48, 10240, 8192) == _lib.VARIANT_TILED
+    assert ops.select_variant(48, 10240, 8192) == _lib.VARIANT_SKINNY  # (64-column narrow tiles: one round on 160 CUs)
+    # against long weight panels (many more tiles than CUs) split-K tiles that fetch B with the
+    # streaming policy win
+    assert ops.select_variant(48, 28672, 8192) == _lib.VARIANT_TILED
     assert ops.select_variant(64, 57344, 8192) == _lib.VARIANT_TILED
     assert ops.select_variant(32, 57344, 8192) == _lib.VARIANT_TILED
     assert ops.select_variant(16, 10240, 8192) == _lib.VARIANT_SKINNY

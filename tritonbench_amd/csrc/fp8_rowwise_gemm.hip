@@ -1504,19 +1504,20 @@ __global__ __launch_bounds__(kPersistWaves * 64) void gemm_skinny_persistent_ker
 // as [slab][row][128 bytes] with the tiled kernel's chunk swizzle; one barrier per step. The
 // four partial 32x32 (x MB) results meet in LDS at the end; wave w finishes columns 8w..8w+7
 // of every 32-row block.
-// SHARED halves the ring depths so that two workgroups fit a CU: for panels of one to two tiles per CU.
 // Workgroup g starts its walk over K at step 5g mod steps and wraps around: with a power-of-two
 // row pitch the rows in flight at one moment would otherwise agree in their low address bits
 // and crowd a few memory channels (measured, M=32, N=K=8192, K loop only: 19.8 -> 13.4 us).
 // ------------------------------------------------------------------------------------
 constexpr int kNarrowKS = 512;
-// SHARED: rings half as deep, so that two workgroups fit a CU (for tile counts between one and two per CU)
-constexpr int narrow_b_dist(bool shared) { return shared ? 2 : 5; }
-constexpr int narrow_a_dist(int MB, bool shared) { return MB == 1 && !shared ? 2 : 1; }
-constexpr size_t narrow_lds_bytes(int MB, bool shared) {
-  return (size_t)(narrow_a_dist(MB, shared) + 1) * MB * 32 * kNarrowKS + (size_t)(narrow_b_dist(shared) + 1) * 32 * kNarrowKS;
+// NB: 32-column blocks per tile (2: 64-column tiles, for panels of one to two 32-column tiles per CU).
+// Steps the loads run ahead of their use: what the 160 KB of LDS allow.
+constexpr int narrow_b_dist(int MB, int NB) { return NB == 1 ? 5 : MB == 1 ? 3 : 2; }
+constexpr int narrow_a_dist(int MB, int NB) { return MB == 1 && NB == 1 ? 2 : 1; }
+constexpr size_t narrow_lds_bytes(int MB, int NB) {
+  return (size_t)(narrow_a_dist(MB, NB) + 1) * MB * 32 * kNarrowKS + (size_t)(narrow_b_dist(MB, NB) + 1) * NB * 32 * kNarrowKS;
 }
-static_assert(narrow_lds_bytes(2, false) <= 160 * 1024 && narrow_lds_bytes(1, true) <= 80 * 1024, "stage rings must fit the LDS");
+static_assert(narrow_lds_bytes(2, 1) <= 160 * 1024 && narrow_lds_bytes(1, 2) <= 160 * 1024 && narrow_lds_bytes(2, 2) <= 160 * 1024,
+              "stage rings must fit the LDS");
 
 // waits until at most VM of this wave's global loads are outstanding (LDS operations are not waited for)
 template <int VM>
@@ -1525,17 +1526,18 @@ __device__ __forceinline__ void wait_loads() {
   __builtin_amdgcn_s_waitcnt(imm);
 }
 
-template <int MB, bool SHARED>
+template <int MB, int NB>
 __global__ __launch_bounds__(512) void gemm_narrow_kernel(GemmParams p) {
-  constexpr int BM = 32 * MB, KS = kNarrowKS, DA = narrow_a_dist(MB, SHARED), DB = narrow_b_dist(SHARED);
+  constexpr int BM = 32 * MB, BN = 32 * NB, KS = kNarrowKS;
+  constexpr int DA = narrow_a_dist(MB, NB), DB = narrow_b_dist(MB, NB);
   constexpr int RA = DA + 1, RB = DB + 1;
-  constexpr int STA = BM * KS, STB = 32 * KS;  // bytes per stage
-  constexpr int LA = BM / 8, LB = 4;           // wave-wide loads per wave and step (8 rows x 128 bytes each)
+  constexpr int STA = BM * KS, STB = BN * KS;  // bytes per stage
+  constexpr int LA = BM / 8, LB = BN / 8;      // wave-wide loads per wave and step (8 rows x 128 bytes each)
   static_assert((DA - 1) * LA < 64 && (DB - 1) * LB < 64, "outstanding-load counts must fit the wait instruction");
   extern __shared__ __attribute__((aligned(1024))) uint8_t lds[];
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-  const int n0 = blockIdx.x * 32;
+  const int n0 = blockIdx.x * BN;
   const int ksteps = p.K / KS;
   const int rot = (int)((blockIdx.x * 5u) % (unsigned)ksteps);
   // a lane's 16 bytes of an 8-row group: row lane/8; LDS position lane%8 holds logical chunk
@@ -1559,28 +1561,33 @@ __global__ __launch_bounds__(512) void gemm_narrow_kernel(GemmParams p) {
       for (int g = 0; g < LA; ++g)
         load_chunk_to_lds<false>(ra, dst + g * 1024, (g & 1) ? a_odd : a_even, (uint32_t)(g * 8) * (uint32_t)p.lda + koff);
     };
-    // this lane's scales and bias, asked for before the loop: row l32 of every block, columns
-    // n0 + 8*wave + 4*half .. +3 (indices clamped; what lies past an edge is never stored)
+    // this lane's scales and bias, asked for before the loop: row l32 of every 32-row block, columns
+    // n0 + 32*jb + 8*wave + 4*half .. +3 of every 32-column block (indices clamped; what lies past an
+    // edge is never stored)
     const int l32 = lane & 31, half = lane >> 5;
     const int nq = n0 + 8 * wave + 4 * half;
-    float sa[MB], sb[4], bias_f[4];
+    float sa[MB], sb[NB][4], bias_f[NB][4];
 #pragma unroll
     for (int i = 0; i < MB; ++i) sa[i] = p.a_scale[min(i * 32 + l32, p.M - 1)];
 #pragma unroll
-    for (int e = 0; e < 4; ++e) {
-      const int ne = min(nq + e, p.N - 1);
-      sb[e] = p.b_scale[ne];
-      bias_f[e] = p.bias ? bf16_to_f32(p.bias[ne]) : 0.0f;
-    }
+    for (int jb = 0; jb < NB; ++jb)
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        const int ne = min(nq + 32 * jb + e, p.N - 1);
+        sb[jb][e] = p.b_scale[ne];
+        bias_f[jb][e] = p.bias ? bf16_to_f32(p.bias[ne]) : 0.0f;
+      }
 #pragma unroll
     for (int s = 0; s < DA; ++s) issue_a(s);
     if (ksteps > DA) wait_loads<(DA - 1) * LA>(); else wait_loads<0>();
     __builtin_amdgcn_s_barrier();
 
-    v16f acc[MB];
+    v16f acc[MB][NB];
     const v16f zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-    for (int i = 0; i < MB; ++i) acc[i] = zero;
+    for (int i = 0; i < MB; ++i)
+#pragma unroll
+      for (int jb = 0; jb < NB; ++jb) acc[i][jb] = zero;
     // fragment of K half sh (64 bytes) of this wave's slab: logical chunks 4*half + 2*sh + {0, 1} of row l32
     int rd[2][2];
 #pragma unroll
@@ -1591,12 +1598,14 @@ __global__ __launch_bounds__(512) void gemm_narrow_kernel(GemmParams p) {
     for (int s = 0; s < ksteps; ++s) {
       issue_a(s + DA);
       const uint8_t* sa_rows = lds + (s % RA) * STA + wave * (BM * kStepK);
-      const uint8_t* sb_rows = lds + RA * STA + (s % RB) * STB + wave * (32 * kStepK);
-      v4i fb[2][2], fa[MB][2][2];
+      const uint8_t* sb_rows = lds + RA * STA + (s % RB) * STB + wave * (BN * kStepK);
+      v4i fb[NB][2][2], fa[MB][2][2];
 #pragma unroll
       for (int sh = 0; sh < 2; ++sh) {
 #pragma unroll
-        for (int j = 0; j < 2; ++j) fb[sh][j] = *(const v4i*)(sb_rows + rd[sh][j]);
+        for (int jb = 0; jb < NB; ++jb)
+#pragma unroll
+          for (int j = 0; j < 2; ++j) fb[jb][sh][j] = *(const v4i*)(sb_rows + jb * 32 * kStepK + rd[sh][j]);
 #pragma unroll
         for (int i = 0; i < MB; ++i)
 #pragma unroll
@@ -1604,13 +1613,16 @@ __global__ __launch_bounds__(512) void gemm_narrow_kernel(GemmParams p) {
       }
 #pragma unroll
       for (int sh = 0; sh < 2; ++sh) {
-        const v8i vb = (v8i){fb[sh][0][0], fb[sh][0][1], fb[sh][0][2], fb[sh][0][3],
-                             fb[sh][1][0], fb[sh][1][1], fb[sh][1][2], fb[sh][1][3]};
 #pragma unroll
-        for (int i = 0; i < MB; ++i) {
-          const v8i va = (v8i){fa[i][sh][0][0], fa[i][sh][0][1], fa[i][sh][0][2], fa[i][sh][0][3],
-                               fa[i][sh][1][0], fa[i][sh][1][1], fa[i][sh][1][2], fa[i][sh][1][3]};
-          acc[i] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(vb, va, acc[i], 0, 0, 0, 0, 0, 0);
+        for (int jb = 0; jb < NB; ++jb) {
+          const v8i vb = (v8i){fb[jb][sh][0][0], fb[jb][sh][0][1], fb[jb][sh][0][2], fb[jb][sh][0][3],
+                               fb[jb][sh][1][0], fb[jb][sh][1][1], fb[jb][sh][1][2], fb[jb][sh][1][3]};
+#pragma unroll
+          for (int i = 0; i < MB; ++i) {
+            const v8i va = (v8i){fa[i][sh][0][0], fa[i][sh][0][1], fa[i][sh][0][2], fa[i][sh][0][3],
+                                 fa[i][sh][1][0], fa[i][sh][1][1], fa[i][sh][1][2], fa[i][sh][1][3]};
+            acc[i][jb] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(vb, va, acc[i][jb], 0, 0, 0, 0, 0, 0);
+          }
         }
       }
       // own loads of A(s+1) have landed (the younger A(s+2) .. A(s+DA) may be in flight); past the barrier
@@ -1620,36 +1632,42 @@ __global__ __launch_bounds__(512) void gemm_narrow_kernel(GemmParams p) {
     }
 
     // ---- the four waves' partial results meet in LDS (the stages are free: last barrier passed)
-    v4f* area = (v4f*)lds;  // [wave][block][q][lane]
+    v4f* area = (v4f*)lds;  // [wave][32x32 block][q][lane]
 #pragma unroll
     for (int i = 0; i < MB; ++i)
 #pragma unroll
-      for (int q = 0; q < 4; ++q)
-        area[((wave * MB + i) * 4 + q) * 64 + lane] = (v4f){acc[i][4 * q], acc[i][4 * q + 1], acc[i][4 * q + 2], acc[i][4 * q + 3]};
+      for (int jb = 0; jb < NB; ++jb)
+#pragma unroll
+        for (int q = 0; q < 4; ++q)
+          area[(((wave * MB + i) * NB + jb) * 4 + q) * 64 + lane] =
+              (v4f){acc[i][jb][4 * q], acc[i][jb][4 * q + 1], acc[i][jb][4 * q + 2], acc[i][jb][4 * q + 3]};
     __syncthreads();
     const bool vec = ((p.ldc & 3) == 0) && ((reinterpret_cast<uintptr_t>(p.c) & 7) == 0);
 #pragma unroll
     for (int i = 0; i < MB; ++i) {
-      v4f sum = area[((0 * MB + i) * 4 + wave) * 64 + lane];
 #pragma unroll
-      for (int w = 1; w < 4; ++w) sum += area[((w * MB + i) * 4 + wave) * 64 + lane];
-      const int m = i * 32 + l32;
-      if (m < p.M && nq < p.N) {
-        float r[4];
+      for (int jb = 0; jb < NB; ++jb) {
+        v4f sum = area[(((0 * MB + i) * NB + jb) * 4 + wave) * 64 + lane];
 #pragma unroll
-        for (int e = 0; e < 4; ++e) {
-          const float t = sum[e] * sa[i];
-          r[e] = p.bias ? __builtin_fmaf(t, sb[e], bias_f[e]) : t * sb[e];
-        }
-        const uint32_t lo = pack_out_x2(r[0], r[1], p.out_f16), hi = pack_out_x2(r[2], r[3], p.out_f16);
-        uint16_t* dst = p.c + (size_t)m * p.ldc + nq;
-        if (vec && nq + 3 < p.N) {
-          *(v2u*)dst = (v2u){lo, hi};
-        } else {
-          dst[0] = (uint16_t)lo;
-          if (nq + 1 < p.N) dst[1] = (uint16_t)(lo >> 16);
-          if (nq + 2 < p.N) dst[2] = (uint16_t)hi;
-          if (nq + 3 < p.N) dst[3] = (uint16_t)(hi >> 16);
+        for (int w = 1; w < 4; ++w) sum += area[(((w * MB + i) * NB + jb) * 4 + wave) * 64 + lane];
+        const int m = i * 32 + l32, n = nq + 32 * jb;
+        if (m < p.M && n < p.N) {
+          float r[4];
+#pragma unroll
+          for (int e = 0; e < 4; ++e) {
+            const float t = sum[e] * sa[i];
+            r[e] = p.bias ? __builtin_fmaf(t, sb[jb][e], bias_f[jb][e]) : t * sb[jb][e];
+          }
+          const uint32_t lo = pack_out_x2(r[0], r[1], p.out_f16), hi = pack_out_x2(r[2], r[3], p.out_f16);
+          uint16_t* dst = p.c + (size_t)m * p.ldc + n;
+          if (vec && n + 3 < p.N) {
+            *(v2u*)dst = (v2u){lo, hi};
+          } else {
+            dst[0] = (uint16_t)lo;
+            if (n + 1 < p.N) dst[1] = (uint16_t)(lo >> 16);
+            if (n + 2 < p.N) dst[2] = (uint16_t)hi;
+            if (n + 3 < p.N) dst[3] = (uint16_t)(hi >> 16);
+          }
         }
       }
     }
@@ -1657,12 +1675,12 @@ __global__ __launch_bounds__(512) void gemm_narrow_kernel(GemmParams p) {
     // ---- loader wave for B: slab `wave - 4` of every step, 8 rows per load
     const int w = wave - 4;
     const __amdgpu_buffer_rsrc_t rb = __builtin_amdgcn_make_buffer_rsrc(
-        const_cast<uint8_t*>(p.b) + (size_t)n0 * p.ldb, 0, (int)((uint32_t)min(p.N - n0, 32) * (uint32_t)p.ldb), 0x00020000);
+        const_cast<uint8_t*>(p.b) + (size_t)n0 * p.ldb, 0, (int)((uint32_t)min(p.N - n0, BN) * (uint32_t)p.ldb), 0x00020000);
     const uint32_t b_even = (uint32_t)ld_row * (uint32_t)p.ldb + chunk_even;
     const uint32_t b_odd = (uint32_t)ld_row * (uint32_t)p.ldb + (chunk_even ^ 64u);
     auto issue_b = [&](int s) {
       if (s >= ksteps) return;
-      uint8_t* dst = lds + RA * STA + (s % RB) * STB + w * (32 * kStepK);
+      uint8_t* dst = lds + RA * STA + (s % RB) * STB + w * (BN * kStepK);
       const uint32_t koff = (uint32_t)step_of(s) * KS + (uint32_t)w * kStepK;
 #pragma unroll
       for (int g = 0; g < LB; ++g)
@@ -2125,15 +2143,17 @@ inline bool narrow_fits(int64_t M, int64_t N, int64_t K) {
   (void)N;
   return M <= 64 && K % 512 == 0;
 }
-// Between one and two tiles per CU, with one block of A: rings half as deep, two workgroups per CU, all
-// tiles resident at once instead of two rounds (measured at K = 8192, M = 32: 22.3 / 23.9 / 24.1 us for
-// N = 10240 / 12288 / 16384; 13.4 us at N = 10240, K = 4096).
-inline bool narrow_shares_cus(int64_t M, int64_t N) {
+// Between one and two 32-column tiles per CU the tiles are 64 columns wide: one round of workgroups on
+// part of the chip instead of two (measured at K = 8192: 18.1 / 19.7 / 23.4 us for N = 10240 / 12288 /
+// 16384 with up to 32 rows of A, 22.8 / 27.2 us for N = 10240 / 16384 with up to 64).
+inline bool narrow_is_wide(int64_t N) {
   const long tiles = (N + 31) / 32;
-  return M <= 32 && tiles > kNumCu && tiles <= 2 * kNumCu;
+  return tiles > kNumCu && tiles <= 2 * kNumCu;
 }
 inline float narrow_cost_us(int64_t M, int64_t N, int64_t K) {
-  if (narrow_shares_cus(M, N)) return 4.5f + (float)K / 1024.0f * 2.4f;
+  // (K = 28672, N = 10240, M = 32: 58.7 us, a lower rate than the shorter rows reach)
+  if (narrow_is_wide(N))
+    return M <= 32 ? 4.0f + (float)N * (float)K / (K > 16384 ? 5.0e6f : 6.3e6f) : 8.0f + (float)N * (float)K / (K > 16384 ? 5.5e6f : 7.0e6f);
   const long tiles = (N + 31) / 32;
   const long rounds = (tiles + kNumCu - 1) / kNumCu;
   return (float)rounds * (M <= 32 ? 3.5f + (float)K / 1024.0f * 1.38f : 4.5f + (float)K / 1024.0f * 1.62f);
@@ -2404,17 +2424,23 @@ int launch_skinny_persistent_steps(const GemmParams& p, hipStream_t s) {
   }
 }
 
-template <int MB, bool SHARED = false>
+template <int MB, int NB>
 int launch_narrow(const GemmParams& p, hipStream_t stream) {
-  constexpr size_t lds_bytes = narrow_lds_bytes(MB, SHARED);
-  auto kern = gemm_narrow_kernel<MB, SHARED>;
+  constexpr size_t lds_bytes = narrow_lds_bytes(MB, NB);
+  auto kern = gemm_narrow_kernel<MB, NB>;
   static bool attr_done[kMaxDevices] = {};
   if (const int st = raise_lds_limit((const void*)kern, lds_bytes, attr_done)) return st;
-  const unsigned grid = (unsigned)((p.N + 31) / 32);
+  const unsigned grid = (unsigned)((p.N + 32 * NB - 1) / (32 * NB));
   hipLaunchKernelGGL(kern, dim3(grid), dim3(512), lds_bytes, stream, p);
   hipError_t e = hipGetLastError();
   if (e != hipSuccess) return fail(MI355X_FP8_ELAUNCH, "narrow-tile kernel launch: %s", hipGetErrorString(e));
   return MI355X_FP8_OK;
+}
+
+// the narrow-tile instantiation for a shape: one or two 32-row blocks of A, 32- or 64-column tiles
+int launch_narrow_for(const GemmParams& p, hipStream_t s) {
+  if (narrow_is_wide(p.N)) return p.M <= 32 ? launch_narrow<1, 2>(p, s) : launch_narrow<2, 2>(p, s);
+  return p.M <= 32 ? launch_narrow<1, 1>(p, s) : launch_narrow<2, 1>(p, s);
 }
 
 }  // namespace
@@ -2540,13 +2566,9 @@ int mi355x_fp8_rowwise_gemm_ex(const void* a, const void* b, const float* a_scal
         if (!narrow_fits(M, N, K))
           return fail(MI355X_FP8_ENOTSUP, "the narrow-tile kernel takes M <= 64 and K in multiples of 512 (got M=%lld, K=%lld)",
                       (long long)M, (long long)K);
-        if (narrow_shares_cus(M, N)) return launch_narrow<1, true>(p, s);
-        return M <= 32 ? launch_narrow<1>(p, s) : launch_narrow<2>(p, s);
+        return launch_narrow_for(p, s);
       }
-      if (!(plan_bits & MI355X_FP8_SKINNY_ONE_TILE) && narrow_preferred(M, N, K)) {
-        if (narrow_shares_cus(M, N)) return launch_narrow<1, true>(p, s);
-        return M <= 32 ? launch_narrow<1>(p, s) : launch_narrow<2>(p, s);
-      }
+      if (!(plan_bits & MI355X_FP8_SKINNY_ONE_TILE) && narrow_preferred(M, N, K)) return launch_narrow_for(p, s);
       if (persistent_skinny_fits(M, N, K) && !(plan_bits & MI355X_FP8_SKINNY_ONE_TILE)) {
         // 16-byte loads of b_scale, 8-byte loads of bias and 8-byte stores of C when everything is aligned for them
         const bool vec = (reinterpret_cast<uintptr_t>(b_scale) & 15) == 0 && (reinterpret_cast<uintptr_t>(bias) & 7) == 0 &&
