@@ -69,7 +69,7 @@ extern "C" {
  * in registers); every other shape runs the general form anyway. */
 #define MI355X_FP8_SKINNY_ONE_TILE      (1 << 8)
 /* Skinny family only: bit 9 pins the narrow-tile form (one workgroup per 32 columns of C owns all
- * of K; M <= 64, K a multiple of 512; "not supported" otherwise). Without a pin the family runs
+ * of K; M <= 64; "not supported" otherwise). Without a pin the family runs
  * whichever of its forms is expected to be fastest. */
 #define MI355X_FP8_SKINNY_NARROW        (2 << 8)
 #define MI355X_FP8_TILED_CONFIG(cfg)    ((((cfg) + 1) & 0xff) << 8)

@@ -1,5 +1,5 @@
-"""Parity of the narrow-tile kernel (M <= 64, K a multiple of 512: one workgroup per 32 columns of
-the output owns all of K) with the CPU oracle, through the C ABI with the kernel pinned, and that
+"""Parity of the narrow-tile kernel (M <= 64: one workgroup per 32 or 64 columns of the output owns
+all of K, in 512-byte steps of which the last may be partial) with the CPU oracle, through the C ABI with the kernel pinned, and that
 the automatic choice takes it where its cost estimate says so. Needs an MI355X."""
 import numpy as np
 import pytest
@@ -59,6 +59,10 @@ SHAPES = [
     # between one and two 32-column tiles per CU: 64-column tiles, with one and two blocks of A
     (32, 16384, 2048, True), (20, 10250, 1024, False), (7, 12288, 512, True), (32, 8224, 4096, False),
     (64, 16384, 1024, False), (40, 9001, 2560, True), (64, 8250, 512, True),
+    # K not in whole 512-byte steps (a partial last step, down to a single 16-byte chunk), not in whole
+    # 128-byte slabs either
+    (32, 64, 528, True), (17, 100, 48, False), (3, 40, 16, True), (40, 1000, 4112, True), (64, 520, 2304, False), (9, 8192, 6672, True),
+    (32, 10240, 1040, False),
 ]
 
 
@@ -72,7 +76,7 @@ def test_narrow_kernel_against_oracle(gpu_device, m, n, k, bias):
     _check_tight(out, xq, wq, xs, ws, b)
 
 
-@pytest.mark.parametrize("m,k", [(32, 512), (19, 2048), (64, 4096), (40, 8192)])
+@pytest.mark.parametrize("m,k", [(32, 512), (19, 2048), (64, 4096), (40, 8192), (32, 2320)])
 def test_exact_integer_case_is_bit_exact(gpu_device, m, k):
     # small integers, unit scales: every partial sum stays below 2^24, so fp32 summation is exact in
     # any order (four waves' partial sums, rotated K order) and the float64 result must come out bit for bit
@@ -182,9 +186,6 @@ def test_shapes_the_kernel_does_not_take_are_refused(gpu_device):
     xq, wq, xs, ws, _ = orc.make_inputs(65, 64, 512, 1.0, False)
     with pytest.raises(NotImplementedError):
         _run(gpu_device, xq, wq, xs, ws, None, NARROW)       # M > 64: not this family at all
-    xq, wq, xs, ws, _ = orc.make_inputs(32, 64, 528, 1.0, False)
-    with pytest.raises(NotImplementedError, match="multiples of 512"):
-        _run(gpu_device, xq, wq, xs, ws, None, NARROW)       # K not in whole steps
 
 
 def test_automatic_choice_runs_it_where_it_is_expected_to_win(gpu_device):

@@ -22,7 +22,7 @@ VARIANT_AUTO = 0
 VARIANT_TILED = 1
 VARIANT_SKINNY = 2
 SKINNY_ONE_TILE = 1 << 8  # skinny family: pins the one-tile-per-workgroup kernel
-SKINNY_NARROW = 2 << 8  # skinny family: pins the narrow-tile kernel (M <= 64, K % 512 == 0)
+SKINNY_NARROW = 2 << 8  # skinny family: pins the narrow-tile kernel (M <= 64)
 
 NUM_TILE_CONFIGS = 4
 NOALLOC_SCRATCH_BYTES = 64 << 20

@@ -1491,7 +1491,7 @@ __global__ __launch_bounds__(kPersistWaves * 64) void gemm_skinny_persistent_ker
 }
 
 // ------------------------------------------------------------------------------------
-// Narrow-tile kernel for M <= 32*MB (MB = 1, 2), K a multiple of 512: one workgroup per 32
+// Narrow-tile kernel for M <= 32*MB (MB = 1, 2): one workgroup per 32
 // columns of C owns all of K, so there are no partial sums and no second launch. It is the
 // form for panels that give every CU at most one such tile (N <= 8192) when A has more rows
 // than the persistent kernel above keeps in registers.
@@ -1538,7 +1538,7 @@ __global__ __launch_bounds__(512) void gemm_narrow_kernel(GemmParams p) {
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int n0 = blockIdx.x * BN;
-  const int ksteps = p.K / KS;
+  const int ksteps = (p.K + KS - 1) / KS;  // the last step may be partial (K is a multiple of 16)
   const int rot = (int)((blockIdx.x * 5u) % (unsigned)ksteps);
   // a lane's 16 bytes of an 8-row group: row lane/8; LDS position lane%8 holds logical chunk
   // position ^ key(row), key = (row >> 1) & 7: for the even groups of a slab that is ld_row >> 1, for
@@ -1546,6 +1546,10 @@ __global__ __launch_bounds__(512) void gemm_narrow_kernel(GemmParams p) {
   const int ld_row = lane >> 3, ld_pc = lane & 7;
   const uint32_t chunk_even = (uint32_t)((ld_pc ^ (ld_row >> 1)) * kChunk);
   auto step_of = [&](int s) { const int t = s + rot; return t >= ksteps ? t - ksteps : t; };
+  // A lane whose 16 bytes lie at or past K (only in the last step of a K that is not a multiple of 512)
+  // asks for an offset outside every descriptor instead: zeros arrive, and the load still counts.
+  constexpr uint32_t kOutside = 0x80000000u;
+  auto lane_part = [&](uint32_t inside, uint32_t chunk, uint32_t k_slab) { return k_slab + chunk < (uint32_t)p.K ? inside : kOutside; };
 
   if (wave < 4) {
     // ---- compute wave: slab `wave` of every step
@@ -1557,9 +1561,10 @@ __global__ __launch_bounds__(512) void gemm_narrow_kernel(GemmParams p) {
       if (s >= ksteps) return;
       uint8_t* dst = lds + (s % RA) * STA + wave * (BM * kStepK);
       const uint32_t koff = (uint32_t)step_of(s) * KS + (uint32_t)wave * kStepK;
+      const uint32_t even = lane_part(a_even, chunk_even, koff), odd = lane_part(a_odd, chunk_even ^ 64u, koff);
 #pragma unroll
       for (int g = 0; g < LA; ++g)
-        load_chunk_to_lds<false>(ra, dst + g * 1024, (g & 1) ? a_odd : a_even, (uint32_t)(g * 8) * (uint32_t)p.lda + koff);
+        load_chunk_to_lds<false>(ra, dst + g * 1024, (g & 1) ? odd : even, (uint32_t)(g * 8) * (uint32_t)p.lda + koff);
     };
     // this lane's scales and bias, asked for before the loop: row l32 of every 32-row block, columns
     // n0 + 32*jb + 8*wave + 4*half .. +3 of every 32-column block (indices clamped; what lies past an
@@ -1682,9 +1687,10 @@ __global__ __launch_bounds__(512) void gemm_narrow_kernel(GemmParams p) {
       if (s >= ksteps) return;
       uint8_t* dst = lds + RA * STA + (s % RB) * STB + w * (BN * kStepK);
       const uint32_t koff = (uint32_t)step_of(s) * KS + (uint32_t)w * kStepK;
+      const uint32_t even = lane_part(b_even, chunk_even, koff), odd = lane_part(b_odd, chunk_even ^ 64u, koff);
 #pragma unroll
       for (int g = 0; g < LB; ++g)
-        load_chunk_to_lds<true>(rb, dst + g * 1024, (g & 1) ? b_odd : b_even, (uint32_t)(g * 8) * (uint32_t)p.ldb + koff);
+        load_chunk_to_lds<true>(rb, dst + g * 1024, (g & 1) ? odd : even, (uint32_t)(g * 8) * (uint32_t)p.ldb + koff);
     };
 #pragma unroll
     for (int s = 0; s < DB; ++s) issue_b(s);
@@ -2136,12 +2142,13 @@ constexpr TileConfig kTileConfigs[kNumTileConfigs] = {
 // four blocks the register budget leaves one workgroup per CU, and a last round of workgroups
 // that fills only part of the CUs streams at that fraction of the rate.
 inline bool persistent_skinny_fits(int64_t M, int64_t N, int64_t K);
-// The narrow-tile kernel: M <= 64, K in whole 512-byte steps. Its cost is one round of workgroups per
+// The narrow-tile kernel: M <= 64. Its cost is one round of workgroups per
 // 256 tiles (measured at N = 8192, cold: 9.8 / 14.3 / 43.0 us for K = 4096 / 8192 / 28672 with up to
 // 32 rows of A, 17.1-17.9 / 49.9 us for K = 8192 / 28672 with up to 64).
 inline bool narrow_fits(int64_t M, int64_t N, int64_t K) {
   (void)N;
-  return M <= 64 && K % 512 == 0;
+  (void)K;
+  return M <= 64;
 }
 // Between one and two 32-column tiles per CU the tiles are 64 columns wide: one round of workgroups on
 // part of the chip instead of two (measured at K = 8192: 18.1 / 19.7 / 23.4 us for N = 10240 / 12288 /
@@ -2564,8 +2571,7 @@ int mi355x_fp8_rowwise_gemm_ex(const void* a, const void* b, const float* a_scal
       // four waves 14.7-15.0 us, six steps in flight 16.4 us, against 14.4 us for this one.)
       if (plan_bits & MI355X_FP8_SKINNY_NARROW) {
         if (!narrow_fits(M, N, K))
-          return fail(MI355X_FP8_ENOTSUP, "the narrow-tile kernel takes M <= 64 and K in multiples of 512 (got M=%lld, K=%lld)",
-                      (long long)M, (long long)K);
+          return fail(MI355X_FP8_ENOTSUP, "the narrow-tile kernel takes M <= 64 (got M=%lld)", (long long)M);
         return launch_narrow_for(p, s);
       }
       if (!(plan_bits & MI355X_FP8_SKINNY_ONE_TILE) && narrow_preferred(M, N, K)) return launch_narrow_for(p, s);
