@@ -49,7 +49,8 @@ extern "C" {
 /* Kernel families. AUTO lets the library pick from (M, N, K). */
 #define MI355X_FP8_VARIANT_AUTO    0
 #define MI355X_FP8_VARIANT_TILED   1  /* LDS-tiled persistent MFMA kernel (compute-bound shapes) */
-#define MI355X_FP8_VARIANT_SKINNY  2  /* in-workgroup split-K streaming kernel (M <= 64 only, HBM-bound) */
+#define MI355X_FP8_VARIANT_SKINNY  2  /* kernels that own all of K per workgroup and stream B (HBM-bound): M <= 64, \
+                                         and M <= 256 where the narrow-tile form below fits */
 
 /*
  * The `variant` argument is a word: bits 0..7 hold the family above; for the tiled family
@@ -68,9 +69,11 @@ extern "C" {
  * the persistent form (one workgroup per CU walks a run of tiles with its share of A resident
  * in registers); every other shape runs the general form anyway. */
 #define MI355X_FP8_SKINNY_ONE_TILE      (1 << 8)
-/* Skinny family only: bit 9 pins the narrow-tile form (one workgroup per 32 columns of C owns all
- * of K; M <= 64; "not supported" otherwise). Without a pin the family runs
- * whichever of its forms is expected to be fastest. */
+/* Skinny family only: bit 9 pins the narrow-tile form (one workgroup per 32 or 64 columns of C owns
+ * all of K). It takes M <= 64 and, in row blocks of 64 with 64-column tiles, 64 < M <= 256 when
+ * ceil(M/64) * ceil(N/64, rounded up to a multiple of 8) <= 256 (one workgroup per CU); "not
+ * supported" otherwise. Without a pin the family runs whichever of its forms is expected to be
+ * fastest. */
 #define MI355X_FP8_SKINNY_NARROW        (2 << 8)
 #define MI355X_FP8_TILED_CONFIG(cfg)    ((((cfg) + 1) & 0xff) << 8)
 #define MI355X_FP8_TILED_SPLITS(s)      (((s) & 0xff) << 16)

@@ -45,6 +45,14 @@ def test_host_side_argument_checks_need_no_gpu():
     assert lib.mi355x_fp8_rowwise_select_variant(32, 2048, 2048) == _lib.VARIANT_SKINNY
     assert lib.mi355x_fp8_rowwise_select_variant(64, 8192, 8192) == _lib.VARIANT_SKINNY  # (its narrow-tile form)
     assert lib.mi355x_fp8_rowwise_select_variant(64, 28672, 8192) == _lib.VARIANT_TILED
+    # (65 .. 256 rows: the narrow-tile form in row blocks where it fits the chip in one round)
+    assert lib.mi355x_fp8_rowwise_select_variant(128, 8192, 8192) == _lib.VARIANT_SKINNY
+    assert lib.mi355x_fp8_rowwise_select_variant(128, 10240, 8192) == _lib.VARIANT_TILED
+    assert lib.mi355x_fp8_rowwise_workspace_bytes(128, 8192, 8192, _lib.VARIANT_AUTO) == 0
+    # the Python mirror of the family's shape rule agrees with the library's choice being possible at all
+    for m, n in ((64, 99999), (65, 16320), (65, 16384), (128, 8192), (128, 8200), (256, 4096), (256, 4160), (257, 64)):
+        if not _lib.skinny_family_takes(m, n):
+            assert lib.mi355x_fp8_rowwise_select_variant(m, n, 1024) == _lib.VARIANT_TILED
     assert lib.mi355x_fp8_rowwise_select_variant(64, 57344, 8192) == _lib.VARIANT_TILED
     assert lib.mi355x_fp8_rowwise_select_variant(0, 8, 16) == _lib.EINVAL
     assert lib.mi355x_fp8_rowwise_select_variant(8, 8, 24) == _lib.ENOTSUP
@@ -77,8 +85,8 @@ def test_workspace_size_follows_the_plan_without_a_gpu():
     assert ws(16, 8192, 8192, _lib.VARIANT_AUTO) == 0
     assert ws(16, 8192, 8192, _lib.VARIANT_SKINNY) == 0
     # few tiles and a long K: split, S * M * N fp32 partial sums
-    auto = ws(128, 8192, 8192, _lib.VARIANT_AUTO)
-    assert auto > 0 and auto % (128 * 8192 * 4) == 0
+    auto = ws(128, 10240, 8192, _lib.VARIANT_AUTO)
+    assert auto > 0 and auto % (128 * 10240 * 4) == 0
     # a pinned split factor is honoured, clipped to the number of 128-byte K steps
     assert ws(256, 256, 1024, _lib.tiled_variant(0, 4)) == 4 * 256 * 256 * 4
     assert ws(256, 256, 1024, _lib.tiled_variant(1, 1)) == 0

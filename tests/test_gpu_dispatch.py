@@ -16,7 +16,8 @@ pytestmark = pytest.mark.gpu
 TOLERANCE = 1.12
 # decode- and small-prefill-sized rows of the Llama-3-70B projection sweep, and the small ragged shape with bias
 SHAPES = [(32, 8192, 8192, False), (64, 8192, 8192, False), (128, 8192, 8192, False), (128, 10240, 8192, False),
-          (32, 10240, 8192, False), (256, 8192, 8192, False), (1000, 3000, 4112, True)]
+          (32, 10240, 8192, False), (256, 8192, 8192, False), (1000, 3000, 4112, True),
+          (128, 8192, 4096, False), (128, 8192, 28672, False), (256, 4096, 8192, False)]
 
 
 def _time_us(dev, m, n, k, bias, variant, sets):
@@ -68,8 +69,9 @@ def test_automatic_choice_is_close_to_the_best_alternative(gpu_device, m, n, k, 
     if m <= 64:
         alternatives["skinny"] = _lib.VARIANT_SKINNY
         alternatives["skinny, one tile per workgroup"] = _lib.VARIANT_SKINNY | _lib.SKINNY_ONE_TILE
-        if k % 512 == 0:
-            alternatives["skinny, narrow tiles"] = _lib.VARIANT_SKINNY | _lib.SKINNY_NARROW
+    # (the narrow-tile form also takes up to 256 rows where 64x64 tiles are one round of workgroups)
+    if _lib.skinny_family_takes(m, n):
+        alternatives["skinny, narrow tiles"] = _lib.VARIANT_SKINNY | _lib.SKINNY_NARROW
     # two rounds over all candidates, the automatic choice first and last: whatever is timed first
     # runs on a colder clock
     # (a third round only if the bound does not hold after two: one noisy replay must not fail the suite)

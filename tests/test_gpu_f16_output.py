@@ -38,7 +38,7 @@ def test_f16_output_every_family(gpu_device, m, n, k, bias):
     want = orc.dequant_matmul(xq, wq, xs, ws, b, out_dtype=torch.float16)
     dev = gpu_device
     d = [None if t is None else t.to(dev) for t in (xq, wq, xs, ws, b)]
-    variants = [_lib.VARIANT_AUTO] + ([_lib.VARIANT_SKINNY] if m <= 64 else [])
+    variants = [_lib.VARIANT_AUTO] + ([_lib.VARIANT_SKINNY] if _lib.skinny_family_takes(m, n) else [])
     variants += [_lib.tiled_variant(cfg, s) for cfg in range(_lib.NUM_TILE_CONFIGS) for s in (1, 3)]
     for variant in variants:
         print(f"case m={m} n={n} k={k} bias={bias} variant={variant:#x}", flush=True)

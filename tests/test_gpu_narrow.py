@@ -1,6 +1,7 @@
-"""Parity of the narrow-tile kernel (M <= 64: one workgroup per 32 or 64 columns of the output owns
-all of K, in 512-byte steps of which the last may be partial) with the CPU oracle, through the C ABI with the kernel pinned, and that
-the automatic choice takes it where its cost estimate says so. Needs an MI355X."""
+"""Parity of the narrow-tile kernel (one workgroup per 32 or 64 columns of the output owns all of K,
+in 512-byte steps of which the last may be partial; M <= 64, and up to 256 rows in row blocks of 64
+where that is one workgroup per CU) with the CPU oracle, through the C ABI with the kernel pinned,
+and that the automatic choice takes it where its cost estimate says so. Needs an MI355X."""
 import numpy as np
 import pytest
 import torch
@@ -63,6 +64,11 @@ SHAPES = [
     # 128-byte slabs either
     (32, 64, 528, True), (17, 100, 48, False), (3, 40, 16, True), (40, 1000, 4112, True), (64, 520, 2304, False), (9, 8192, 6672, True),
     (32, 10240, 1040, False),
+    # more than 64 rows: row blocks of 64 with 64-column tiles, the workgroups of a tile side by side on
+    # one XCD; ragged last row block (1, 32 and 36 rows), ragged last tile, fewer tiles than XCDs, a
+    # grid of exactly 256 workgroups, partial last K step
+    (65, 64, 512, True), (128, 8192, 1024, False), (100, 1000, 2048, True), (96, 4100, 1536, False),
+    (256, 4096, 1024, True), (192, 5000, 512, False), (129, 200, 4112, True), (128, 7168, 2320, False),
 ]
 
 
@@ -76,7 +82,7 @@ def test_narrow_kernel_against_oracle(gpu_device, m, n, k, bias):
     _check_tight(out, xq, wq, xs, ws, b)
 
 
-@pytest.mark.parametrize("m,k", [(32, 512), (19, 2048), (64, 4096), (40, 8192), (32, 2320)])
+@pytest.mark.parametrize("m,k", [(32, 512), (19, 2048), (64, 4096), (40, 8192), (32, 2320), (120, 2048), (190, 1040)])
 def test_exact_integer_case_is_bit_exact(gpu_device, m, k):
     # small integers, unit scales: every partial sum stays below 2^24, so fp32 summation is exact in
     # any order (four waves' partial sums, rotated K order) and the float64 result must come out bit for bit
@@ -182,10 +188,47 @@ def test_graph_capture_replays_match_eager(gpu_device):
         assert torch.equal(out, eager)
 
 
+def test_one_hot_positions_with_row_blocks(gpu_device):
+    # the same walk with three row blocks and 40 tiles (five rounds of the XCDs): a wrong row-block or
+    # tile assignment of a workgroup shows as a misplaced one
+    m, n, k = 150, 2500, 4096
+    ka = (np.arange(m) * 517 + 5) % k
+    kb = (np.arange(n) * 131 + 2) % k
+    kb[: m * 8] = np.repeat(ka, 8)
+    a = np.zeros((m, k), np.float32)
+    b = np.zeros((n, k), np.float32)
+    a[np.arange(m), ka] = 1.0
+    b[np.arange(n), kb] = 1.0
+    out = _run(gpu_device, torch.from_numpy(a).to(torch.float8_e4m3fn), torch.from_numpy(b).to(torch.float8_e4m3fn),
+               torch.ones(m), torch.ones(n), None, NARROW)
+    want = (ka[:, None] == kb[None, :]).astype(np.float32)
+    assert np.array_equal(out.float().numpy(), want)
+
+
+def test_row_blocks_keep_to_their_rows_of_an_embedded_output(gpu_device):
+    m, n, k = 130, 700, 1024
+    xq, wq, xs, ws, b = orc.make_inputs(m, n, k, 1.0, True)
+    want = orc.dequant_matmul(xq, wq, xs, ws, b)
+    dev = gpu_device
+    c_buf = torch.full((m + 2, n + 25), -77.0, dtype=torch.bfloat16, device=dev)
+    c_view = c_buf[1:m + 1, 7:7 + n]
+    ops.fp8_gemm_rowwise(xq.to(dev), wq.to(dev), xs.to(dev), ws.to(dev), bias=b.to(dev), out=c_view, variant=NARROW)
+    torch.cuda.synchronize()
+    torch.testing.assert_close(c_view.cpu(), want, rtol=RTOL, atol=ATOL)
+    mask = torch.ones_like(c_buf, dtype=torch.bool)
+    mask[1:m + 1, 7:7 + n] = False
+    assert torch.all(c_buf[mask] == -77.0)
+
+
 def test_shapes_the_kernel_does_not_take_are_refused(gpu_device):
-    xq, wq, xs, ws, _ = orc.make_inputs(65, 64, 512, 1.0, False)
-    with pytest.raises(NotImplementedError):
-        _run(gpu_device, xq, wq, xs, ws, None, NARROW)       # M > 64: not this family at all
+    # more than 64 rows are taken only where 64x64 tiles give every CU at most one workgroup
+    for m, n in ((257, 64), (128, 8200), (256, 4160), (65, 16384)):
+        assert not _lib.skinny_family_takes(m, n)
+        xq, wq, xs, ws, _ = orc.make_inputs(m, n, 512, 1.0, False)
+        with pytest.raises(NotImplementedError):
+            _run(gpu_device, xq, wq, xs, ws, None, NARROW)
+        with pytest.raises(NotImplementedError):
+            _run(gpu_device, xq, wq, xs, ws, None, _lib.VARIANT_SKINNY)
 
 
 def test_automatic_choice_runs_it_where_it_is_expected_to_win(gpu_device):
@@ -197,3 +240,12 @@ def test_automatic_choice_runs_it_where_it_is_expected_to_win(gpu_device):
     auto = _run(gpu_device, xq, wq, xs, ws, b, _lib.VARIANT_AUTO)
     pinned = _run(gpu_device, xq, wq, xs, ws, b, NARROW)
     assert torch.equal(auto, pinned)  # the same kernel: bit-identical
+    # 128 x 8192 x 8192: two row blocks, 256 workgroups, no partial sums in a workspace
+    assert ops.select_variant(128, 8192, 8192) == _lib.VARIANT_SKINNY
+    assert _lib.load().mi355x_fp8_rowwise_workspace_bytes(128, 8192, 8192, _lib.VARIANT_AUTO) == 0
+    assert ops.select_variant(128, 10240, 8192) == _lib.VARIANT_TILED
+    xq, wq, xs, ws, b = orc.make_inputs(128, 8192, 2048, 0.02, True)
+    assert ops.select_variant(128, 8192, 2048) == _lib.VARIANT_SKINNY
+    auto = _run(gpu_device, xq, wq, xs, ws, b, _lib.VARIANT_AUTO)
+    pinned = _run(gpu_device, xq, wq, xs, ws, b, NARROW)
+    assert torch.equal(auto, pinned)

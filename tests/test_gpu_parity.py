@@ -63,7 +63,7 @@ def test_golden_fixtures(gpu_device):
         bias = torch.from_numpy(z["bias"].view(np.int16)).view(torch.bfloat16) if case["bias"] else None
         want = torch.from_numpy(z["c"].view(np.int16)).view(torch.bfloat16)
         for variant in VARIANTS:
-            if variant == _lib.VARIANT_SKINNY and case["m"] > 64:
+            if variant == _lib.VARIANT_SKINNY and not _lib.skinny_family_takes(case["m"], case["n"]):
                 continue
             print(f"golden {case['name']} variant {variant}", flush=True)
             out = _run(gpu_device, xq, wq, xs, ws, bias, variant)
@@ -83,8 +83,8 @@ SMALL_SHAPES = [
 @pytest.mark.parametrize("m,n,k,bias", SMALL_SHAPES)
 @pytest.mark.parametrize("variant", VARIANTS)
 def test_seeded_shapes_against_oracle(gpu_device, m, n, k, bias, variant):
-    if variant == _lib.VARIANT_SKINNY and m > 64:
-        pytest.skip("skinny variant covers M <= 64")
+    if variant == _lib.VARIANT_SKINNY and not _lib.skinny_family_takes(m, n):
+        pytest.skip("the skinny family does not take this shape")
     print(f"case m={m} n={n} k={k} bias={bias} variant={variant}", flush=True)
     xq, wq, xs, ws, b = orc.make_inputs(m, n, k, 1.0, bias)
     want = orc.dequant_matmul(xq, wq, xs, ws, b)
@@ -314,7 +314,7 @@ def test_unsupported_and_invalid_arguments_raise(gpu_device):
     with pytest.raises(NotImplementedError, match="multiple of 16"):
         ops.fp8_gemm_rowwise(f8(16, 24), f8(16, 24), torch.ones(16, device=dev), torch.ones(16, device=dev))
     with pytest.raises(NotImplementedError, match="skinny"):
-        ops.fp8_gemm_rowwise(f8(128, 32), f8(16, 32), torch.ones(128, device=dev), torch.ones(16, device=dev),
+        ops.fp8_gemm_rowwise(f8(320, 32), f8(16, 32), torch.ones(320, device=dev), torch.ones(16, device=dev),
                              variant=_lib.VARIANT_SKINNY)
     with pytest.raises(TypeError):
         ops.fp8_gemm_rowwise(torch.zeros(16, 16, device=dev), f8(16, 16), torch.ones(16, device=dev), torch.ones(16, device=dev))
@@ -344,6 +344,11 @@ def test_dispatch_is_pinned(gpu_device):
     assert ops.select_variant(64, 57344, 8192) == _lib.VARIANT_TILED
     assert ops.select_variant(32, 57344, 8192) == _lib.VARIANT_TILED
     assert ops.select_variant(16, 10240, 8192) == _lib.VARIANT_SKINNY
+    # 65 .. 256 rows: the narrow-tile form in row blocks where that is one workgroup per CU and K is not too long
+    assert ops.select_variant(128, 8192, 8192) == _lib.VARIANT_SKINNY
+    assert ops.select_variant(128, 8192, 28672) == _lib.VARIANT_TILED
+    assert ops.select_variant(128, 10240, 8192) == _lib.VARIANT_TILED
+    assert ops.select_variant(512, 8192, 8192) == _lib.VARIANT_TILED
 
 
 def test_graph_capture_replays_match_eager(gpu_device):

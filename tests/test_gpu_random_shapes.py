@@ -31,7 +31,7 @@ def test_random_shapes_every_plan(gpu_device, m, n, k, bias):
     dev = gpu_device
     d = [None if t is None else t.to(dev) for t in (xq, wq, xs, ws, b)]
     variants = [_lib.VARIANT_AUTO]
-    if m <= 64:
+    if _lib.skinny_family_takes(m, n):
         variants.append(_lib.VARIANT_SKINNY)
     rng = np.random.default_rng(m * 7919 + n * 31 + k)
     for cfg in range(_lib.NUM_TILE_CONFIGS):

@@ -22,7 +22,16 @@ VARIANT_AUTO = 0
 VARIANT_TILED = 1
 VARIANT_SKINNY = 2
 SKINNY_ONE_TILE = 1 << 8  # skinny family: pins the one-tile-per-workgroup kernel
-SKINNY_NARROW = 2 << 8  # skinny family: pins the narrow-tile kernel (M <= 64)
+SKINNY_NARROW = 2 << 8  # skinny family: pins the narrow-tile kernel (the shapes `skinny_family_takes`)
+
+
+def skinny_family_takes(m: int, n: int) -> bool:
+    """Whether VARIANT_SKINNY accepts an M x N output (it answers "not supported" otherwise): up to
+    64 rows always; up to 256 rows where 64x64 tiles in row blocks of 64, the tile count rounded up to
+    a multiple of 8, are at most one workgroup per CU."""
+    if m <= 64:
+        return True
+    return m <= 256 and -(-m // 64) * ((-(-n // 64) + 7) // 8 * 8) <= 256
 
 NUM_TILE_CONFIGS = 4
 NOALLOC_SCRATCH_BYTES = 64 << 20

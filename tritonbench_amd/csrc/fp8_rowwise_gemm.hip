@@ -1537,9 +1537,20 @@ __global__ __launch_bounds__(512) void gemm_narrow_kernel(GemmParams p) {
   extern __shared__ __attribute__((aligned(1024))) uint8_t lds[];
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-  const int n0 = blockIdx.x * BN;
+  // More than BM rows of A: a workgroup per tile and row block. The workgroups of one tile sit next to
+  // each other on one XCD (workgroup ids go round the XCDs), so the tile's rows of B come from HBM once
+  // and from that XCD's L2 for the others.
+  const int row_blocks = (p.M + BM - 1) / BM;
+  int tile = blockIdx.x, row_block = 0;
+  if (row_blocks > 1) {
+    const int slot = blockIdx.x / kNumXcd;
+    row_block = slot % row_blocks;
+    tile = (slot / row_blocks) * kNumXcd + (blockIdx.x % kNumXcd);
+    if (tile * BN >= p.N) return;  // (the grid is rounded up to whole rounds of the XCDs)
+  }
+  const int n0 = tile * BN, m0 = row_block * BM;
   const int ksteps = (p.K + KS - 1) / KS;  // the last step may be partial (K is a multiple of 16)
-  const int rot = (int)((blockIdx.x * 5u) % (unsigned)ksteps);
+  const int rot = (int)(((unsigned)tile * 5u) % (unsigned)ksteps);
   // a lane's 16 bytes of an 8-row group: row lane/8; LDS position lane%8 holds logical chunk
   // position ^ key(row), key = (row >> 1) & 7: for the even groups of a slab that is ld_row >> 1, for
   // the odd ones 4 more, which flips bit 6 of the byte offset
@@ -1554,7 +1565,7 @@ __global__ __launch_bounds__(512) void gemm_narrow_kernel(GemmParams p) {
   if (wave < 4) {
     // ---- compute wave: slab `wave` of every step
     const __amdgpu_buffer_rsrc_t ra = __builtin_amdgcn_make_buffer_rsrc(
-        const_cast<uint8_t*>(p.a), 0, (int)((uint32_t)min(p.M, BM) * (uint32_t)p.lda), 0x00020000);
+        const_cast<uint8_t*>(p.a) + (size_t)m0 * p.lda, 0, (int)((uint32_t)min(p.M - m0, BM) * (uint32_t)p.lda), 0x00020000);
     const uint32_t a_even = (uint32_t)ld_row * (uint32_t)p.lda + chunk_even;
     const uint32_t a_odd = (uint32_t)ld_row * (uint32_t)p.lda + (chunk_even ^ 64u);
     auto issue_a = [&](int s) {
@@ -1573,7 +1584,7 @@ __global__ __launch_bounds__(512) void gemm_narrow_kernel(GemmParams p) {
     const int nq = n0 + 8 * wave + 4 * half;
     float sa[MB], sb[NB][4], bias_f[NB][4];
 #pragma unroll
-    for (int i = 0; i < MB; ++i) sa[i] = p.a_scale[min(i * 32 + l32, p.M - 1)];
+    for (int i = 0; i < MB; ++i) sa[i] = p.a_scale[min(m0 + i * 32 + l32, p.M - 1)];
 #pragma unroll
     for (int jb = 0; jb < NB; ++jb)
 #pragma unroll
@@ -1655,7 +1666,7 @@ __global__ __launch_bounds__(512) void gemm_narrow_kernel(GemmParams p) {
         v4f sum = area[(((0 * MB + i) * NB + jb) * 4 + wave) * 64 + lane];
 #pragma unroll
         for (int w = 1; w < 4; ++w) sum += area[(((w * MB + i) * NB + jb) * 4 + wave) * 64 + lane];
-        const int m = i * 32 + l32, n = nq + 32 * jb;
+        const int m = m0 + i * 32 + l32, n = nq + 32 * jb;
         if (m < p.M && n < p.N) {
           float r[4];
 #pragma unroll
@@ -2145,10 +2156,15 @@ inline bool persistent_skinny_fits(int64_t M, int64_t N, int64_t K);
 // The narrow-tile kernel: M <= 64. Its cost is one round of workgroups per
 // 256 tiles (measured at N = 8192, cold: 9.8 / 14.3 / 43.0 us for K = 4096 / 8192 / 28672 with up to
 // 32 rows of A, 17.1-17.9 / 49.9 us for K = 8192 / 28672 with up to 64).
+// Up to 256 rows of A it runs 64x64 tiles in row blocks of 64 where that is one round of workgroups,
+// one per CU (measured: 13.7 / 21.5 / 67.6 us for K = 4096 / 8192 / 28672 at M = 128, N = 8192;
+// 20.2-20.4 us for M = 128 .. 256 at N = 4096, K = 8192).
+constexpr int kNarrowMaxM = 256;
 inline bool narrow_fits(int64_t M, int64_t N, int64_t K) {
-  (void)N;
   (void)K;
-  return M <= 64;
+  if (M <= kSkinnyMaxM) return true;
+  const long tiles = ((N + 63) / 64 + kNumXcd - 1) / kNumXcd * kNumXcd, row_blocks = (M + 63) / 64;
+  return M <= kNarrowMaxM && tiles * row_blocks <= kNumCu;
 }
 // Between one and two 32-column tiles per CU the tiles are 64 columns wide: one round of workgroups on
 // part of the chip instead of two (measured at K = 8192: 18.1 / 19.7 / 23.4 us for N = 10240 / 12288 /
@@ -2158,6 +2174,7 @@ inline bool narrow_is_wide(int64_t N) {
   return tiles > kNumCu && tiles <= 2 * kNumCu;
 }
 inline float narrow_cost_us(int64_t M, int64_t N, int64_t K) {
+  if (M > kSkinnyMaxM) return 6.0f + (float)K / 1024.0f * (K > 16384 ? 2.15f : 1.9f);
   // (K = 28672, N = 10240, M = 32: 58.7 us, a lower rate than the shorter rows reach)
   if (narrow_is_wide(N))
     return M <= 32 ? 4.0f + (float)N * (float)K / (K > 16384 ? 5.0e6f : 6.3e6f) : 8.0f + (float)N * (float)K / (K > 16384 ? 5.5e6f : 7.0e6f);
@@ -2184,9 +2201,11 @@ inline float skinny_streaming_cost_us(int64_t M, int64_t N, int64_t K) {
 }
 // the cheapest member of the M <= 64 family: streaming (persistent or one tile per workgroup) or narrow tiles
 inline bool narrow_preferred(int64_t M, int64_t N, int64_t K) {
+  if (M > kSkinnyMaxM) return narrow_fits(M, N, K);  // (the streaming kernels stop at 64 rows)
   return narrow_fits(M, N, K) && narrow_cost_us(M, N, K) < skinny_streaming_cost_us(M, N, K);
 }
 inline float skinny_cost_us(int64_t M, int64_t N, int64_t K) {
+  if (M > kSkinnyMaxM && !narrow_fits(M, N, K)) return 1e30f;
   return narrow_preferred(M, N, K) ? narrow_cost_us(M, N, K) : skinny_streaming_cost_us(M, N, K);
 }
 constexpr int kMaxSplits = 16;
@@ -2437,7 +2456,10 @@ int launch_narrow(const GemmParams& p, hipStream_t stream) {
   auto kern = gemm_narrow_kernel<MB, NB>;
   static bool attr_done[kMaxDevices] = {};
   if (const int st = raise_lds_limit((const void*)kern, lds_bytes, attr_done)) return st;
-  const unsigned grid = (unsigned)((p.N + 32 * NB - 1) / (32 * NB));
+  const unsigned tiles = (unsigned)((p.N + 32 * NB - 1) / (32 * NB));
+  const unsigned row_blocks = (unsigned)((p.M + 32 * MB - 1) / (32 * MB));
+  // (with row blocks the kernel deals tiles out per XCD: whole rounds of the XCDs)
+  const unsigned grid = row_blocks == 1 ? tiles : (tiles + kNumXcd - 1) / kNumXcd * kNumXcd * row_blocks;
   hipLaunchKernelGGL(kern, dim3(grid), dim3(512), lds_bytes, stream, p);
   hipError_t e = hipGetLastError();
   if (e != hipSuccess) return fail(MI355X_FP8_ELAUNCH, "narrow-tile kernel launch: %s", hipGetErrorString(e));
@@ -2446,6 +2468,7 @@ int launch_narrow(const GemmParams& p, hipStream_t stream) {
 
 // the narrow-tile instantiation for a shape: one or two 32-row blocks of A, 32- or 64-column tiles
 int launch_narrow_for(const GemmParams& p, hipStream_t s) {
+  if (p.M > 64) return launch_narrow<2, 2>(p, s);
   if (narrow_is_wide(p.N)) return p.M <= 32 ? launch_narrow<1, 2>(p, s) : launch_narrow<2, 2>(p, s);
   return p.M <= 32 ? launch_narrow<1, 1>(p, s) : launch_narrow<2, 1>(p, s);
 }
@@ -2465,7 +2488,8 @@ int mi355x_fp8_rowwise_select_variant(int64_t M, int64_t N, int64_t K) {
   // K where the tiles are few) is expected to beat it: from two 16-row blocks of A up on most
   // shapes, with one block on the longest weight panels. Up to 8 rows the streaming kernel was
   // never behind on any measured shape, so there the estimates are not consulted.
-  if (M > kSkinnyMaxM) return MI355X_FP8_VARIANT_TILED;
+  // (above 64 rows the family's only member is the narrow-tile kernel in row blocks, where it fits)
+  if (M > kSkinnyMaxM && !narrow_fits(M, N, K)) return MI355X_FP8_VARIANT_TILED;
   if (M <= 8) return MI355X_FP8_VARIANT_SKINNY;
   return plan_tiled(M, N, K, -1, 0, kMaxSplits).cost_us < skinny_cost_us(M, N, K) ? MI355X_FP8_VARIANT_TILED
                                                                                  : MI355X_FP8_VARIANT_SKINNY;
@@ -2513,7 +2537,7 @@ int mi355x_fp8_rowwise_gemm_ex(const void* a, const void* b, const float* a_scal
   variant &= 0xff;
   if (variant == MI355X_FP8_VARIANT_AUTO) {
     variant = mi355x_fp8_rowwise_select_variant(M, N, K);
-    if (variant == MI355X_FP8_VARIANT_TILED && M <= kSkinnyMaxM) {
+    if (variant == MI355X_FP8_VARIANT_TILED && (M <= kSkinnyMaxM || narrow_fits(M, N, K))) {
       // the choice assumed the plan's workspace; without it the plan changes and may lose
       const TiledPlan plan = plan_from_variant(M, N, K, plan_bits, kMaxSplits);
       const size_t need = plan.splits > 1 ? (size_t)plan.splits * M * N * sizeof(float) : 0;
@@ -2522,8 +2546,10 @@ int mi355x_fp8_rowwise_gemm_ex(const void* a, const void* b, const float* a_scal
         variant = MI355X_FP8_VARIANT_SKINNY;
     }
   }
-  if (variant == MI355X_FP8_VARIANT_SKINNY && M > kSkinnyMaxM)
-    return fail(MI355X_FP8_ENOTSUP, "skinny variant handles M <= %d (got %lld)", kSkinnyMaxM, (long long)M);
+  if (variant == MI355X_FP8_VARIANT_SKINNY && M > kSkinnyMaxM && !narrow_fits(M, N, K))
+    return fail(MI355X_FP8_ENOTSUP,
+                "skinny variant handles M <= %d, and M <= %d where 64x64 tiles give every CU at most one (got %lldx%lld)",
+                kSkinnyMaxM, kNarrowMaxM, (long long)M, (long long)N);
 
   GemmParams p;
   p.a = (const uint8_t*)a; p.b = (const uint8_t*)b;
@@ -2571,9 +2597,12 @@ int mi355x_fp8_rowwise_gemm_ex(const void* a, const void* b, const float* a_scal
       // four waves 14.7-15.0 us, six steps in flight 16.4 us, against 14.4 us for this one.)
       if (plan_bits & MI355X_FP8_SKINNY_NARROW) {
         if (!narrow_fits(M, N, K))
-          return fail(MI355X_FP8_ENOTSUP, "the narrow-tile kernel takes M <= 64 (got M=%lld)", (long long)M);
+          return fail(MI355X_FP8_ENOTSUP,
+                      "the narrow-tile kernel takes M <= %d, and M <= %d where 64x64 tiles give every CU at most one (got %lldx%lld)",
+                      kSkinnyMaxM, kNarrowMaxM, (long long)M, (long long)N);
         return launch_narrow_for(p, s);
       }
+      if (M > kSkinnyMaxM) return launch_narrow_for(p, s);
       if (!(plan_bits & MI355X_FP8_SKINNY_ONE_TILE) && narrow_preferred(M, N, K)) return launch_narrow_for(p, s);
       if (persistent_skinny_fits(M, N, K) && !(plan_bits & MI355X_FP8_SKINNY_ONE_TILE)) {
         // 16-byte loads of b_scale, 8-byte loads of bias and 8-byte stores of C when everything is aligned for them
