@@ -64,11 +64,14 @@ SHAPES = [
     # 128-byte slabs either
     (32, 64, 528, True), (17, 100, 48, False), (3, 40, 16, True), (40, 1000, 4112, True), (64, 520, 2304, False), (9, 8192, 6672, True),
     (32, 10240, 1040, False),
-    # more than 64 rows: row blocks of 64 with 64-column tiles, the workgroups of a tile side by side on
-    # one XCD; ragged last row block (1, 32 and 36 rows), ragged last tile, fewer tiles than XCDs, a
-    # grid of exactly 256 workgroups, partial last K step
+    # row blocks (the workgroups of a tile side by side on one XCD) in every tile size: 32x32 tiles with
+    # two to five blocks, 64x32 with two and four, 64x64 with two to four; ragged last row block (1, 4, 32
+    # and 36 rows), ragged last tile, fewer tiles than XCDs, grids of exactly 256 workgroups, partial last
+    # K step; and 64 rows in one block where two would be too many workgroups
     (65, 64, 512, True), (128, 8192, 1024, False), (100, 1000, 2048, True), (96, 4100, 1536, False),
     (256, 4096, 1024, True), (192, 5000, 512, False), (129, 200, 4112, True), (128, 7168, 2320, False),
+    (128, 4096, 1024, True), (256, 2000, 528, False), (100, 3000, 1040, True), (64, 7000, 1024, True),
+    (64, 4096, 1536, False),
 ]
 
 

@@ -140,7 +140,7 @@ def test_split_k_exact_integer_case_is_bit_exact(gpu_device, config):
 def test_workspace_rules(gpu_device):
     dev = gpu_device
     lib = _lib.load()
-    m, n, k = 128, 2048, 8192
+    m, n, k = 300, 2048, 8192
     xq, wq, xs, ws, _ = orc.make_inputs(m, n, k, 1.0, False)
     dxq, dwq, dxs, dws = (t.to(dev) for t in (xq, wq, xs, ws))
     want = orc.dequant_matmul(xq, wq, xs, ws, None)

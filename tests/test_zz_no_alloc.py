@@ -14,7 +14,7 @@ from tritonbench_amd import _lib
 
 # (m, n, k, bias): shapes whose automatic plan splits K, i.e. really uses the scratch buffer;
 # the second is smaller in every dimension and leaves stale partial sums of the first behind it
-SPLIT_SHAPES = [(128, 1536, 8192, True), (96, 640, 4096, False)]
+SPLIT_SHAPES = [(320, 1536, 8192, True), (264, 640, 4096, False)]
 # a shape whose plan needs no scratch at all, after the two above
 PLAIN_SHAPE = (512, 1024, 512, True)
 

@@ -17,8 +17,9 @@
 //                            split K between them and reduce through LDS; B is streamed once.
 //   gemm_skinny_persistent_kernel  M <= 16 (M <= 32 at K = 4096): one 16-wave workgroup per CU keeps
 //                            its share of A in registers and walks 16-row tiles of B.
-//   gemm_narrow_kernel       M <= 64, K in 512-byte steps, at most one 32-column tile per CU: a workgroup
-//                            owns all of K (no split, no second launch); separate waves fetch A and B.
+//   gemm_narrow_kernel       M <= 64 (M <= 256 in row blocks), K in 512-byte steps, at most one 32- or
+//                            64-column tile per CU: a workgroup owns all of K (no split, no second
+//                            launch); separate waves fetch A and B.
 //   quantize_rows_*_kernel   row-wise e4m3fn quantiser (amax, scale, convert), one row per workgroup.
 //   fused_rowwise_quant_kernel  RMSNorm or SiLU-mul of bf16 rows followed by the same quantiser, one pass.
 //
@@ -1491,10 +1492,10 @@ __global__ __launch_bounds__(kPersistWaves * 64) void gemm_skinny_persistent_ker
 }
 
 // ------------------------------------------------------------------------------------
-// Narrow-tile kernel for M <= 32*MB (MB = 1, 2): one workgroup per 32
-// columns of C owns all of K, so there are no partial sums and no second launch. It is the
-// form for panels that give every CU at most one such tile (N <= 8192) when A has more rows
-// than the persistent kernel above keeps in registers.
+// Narrow-tile kernel: one workgroup per tile of 32*MB rows and 32*NB columns of C (MB, NB = 1, 2)
+// owns all of K, so there are no partial sums and no second launch. It is the form for shapes
+// that give every CU at most one such tile when A has more rows than the persistent kernel
+// above keeps in registers: up to 64 rows on any panel, up to 256 in row blocks.
 //
 // Eight waves. A K step is 512 bytes: wave w of the first four fetches and multiplies the
 // step's w-th 128-byte slab of A (rows of A are L2 hits: a short queue, DA steps ahead), wave
@@ -2153,12 +2154,14 @@ constexpr TileConfig kTileConfigs[kNumTileConfigs] = {
 // four blocks the register budget leaves one workgroup per CU, and a last round of workgroups
 // that fills only part of the CUs streams at that fraction of the rate.
 inline bool persistent_skinny_fits(int64_t M, int64_t N, int64_t K);
-// The narrow-tile kernel: M <= 64. Its cost is one round of workgroups per
+// The narrow-tile kernel. With all rows in one workgroup (M <= 64) its cost is one round of workgroups per
 // 256 tiles (measured at N = 8192, cold: 9.8 / 14.3 / 43.0 us for K = 4096 / 8192 / 28672 with up to
 // 32 rows of A, 17.1-17.9 / 49.9 us for K = 8192 / 28672 with up to 64).
-// Up to 256 rows of A it runs 64x64 tiles in row blocks of 64 where that is one round of workgroups,
-// one per CU (measured: 13.7 / 21.5 / 67.6 us for K = 4096 / 8192 / 28672 at M = 128, N = 8192;
-// 20.2-20.4 us for M = 128 .. 256 at N = 4096, K = 8192).
+// Up to 256 rows of A it runs in row blocks where that is one round of workgroups, one per CU
+// (measured, K = 8192 unless given: 64x64 tiles 13.7 / 21.5 / 67.6 us for K = 4096 / 8192 / 28672 at
+// M = 128, N = 8192; 64x32 tiles 10.7 / 16.0 / 24.2 us for K = 4096 / 8192 / 14336 at M = 128, N = 4096,
+// 14.0 us at 192 x 1536; 32x32 tiles 12.6 us at 64 x 4096, 11.3 us at 128 x 2048, 11.0 us at 64 x 1024,
+// 8.3 us at 64 x 4096 x 4096, 37.1 us at 64 x 4096 x 28672).
 constexpr int kNarrowMaxM = 256;
 inline bool narrow_fits(int64_t M, int64_t N, int64_t K) {
   (void)K;
@@ -2173,8 +2176,34 @@ inline bool narrow_is_wide(int64_t N) {
   const long tiles = (N + 31) / 32;
   return tiles > kNumCu && tiles <= 2 * kNumCu;
 }
+// The form for a shape: 32-row blocks of A per workgroup (the rows beyond them go to further row
+// blocks) and 32-column blocks per tile. Up to 32 rows, and up to 64 on panels too wide for row
+// blocks: all rows in one workgroup, 64-column tiles between one and two 32-column tiles per CU.
+// Otherwise the smallest tile whose row blocks are one round of workgroups: more CUs at work, and
+// less to deliver into each one's LDS.
+struct NarrowForm {
+  int mb, nb;
+};
+inline long narrow_workgroups(int64_t M, int64_t N, NarrowForm f) {
+  const long tiles = (N + 32 * f.nb - 1) / (32 * f.nb), row_blocks = (M + 32 * f.mb - 1) / (32 * f.mb);
+  return row_blocks == 1 ? tiles : (tiles + kNumXcd - 1) / kNumXcd * kNumXcd * row_blocks;
+}
+inline NarrowForm narrow_form(int64_t M, int64_t N) {
+  if (M <= 32) return {1, narrow_is_wide(N) ? 2 : 1};
+  static const NarrowForm by_size[3] = {{1, 1}, {2, 1}, {2, 2}};
+  for (const NarrowForm f : by_size)
+    if (narrow_workgroups(M, N, f) <= kNumCu) return f;
+  return {2, narrow_is_wide(N) ? 2 : 1};  // (M <= 64: several rounds of workgroups)
+}
 inline float narrow_cost_us(int64_t M, int64_t N, int64_t K) {
-  if (M > kSkinnyMaxM) return 6.0f + (float)K / 1024.0f * (K > 16384 ? 2.15f : 1.9f);
+  const NarrowForm f = narrow_form(M, N);
+  if (M > 32 * f.mb) {  // row blocks, one round
+    const float k1024 = (float)K / 1024.0f;
+    if (f.nb == 2) return 6.0f + k1024 * (K > 16384 ? 2.15f : 1.9f);
+    const float share = (float)narrow_workgroups(M, N, f) / (float)kNumCu;  // of the CUs at work
+    if (f.mb == 2) return 5.4f + k1024 * (0.75f + 0.575f * share);
+    return 3.5f + k1024 * (0.9f + 0.25f * share);
+  }
   // (K = 28672, N = 10240, M = 32: 58.7 us, a lower rate than the shorter rows reach)
   if (narrow_is_wide(N))
     return M <= 32 ? 4.0f + (float)N * (float)K / (K > 16384 ? 5.0e6f : 6.3e6f) : 8.0f + (float)N * (float)K / (K > 16384 ? 5.5e6f : 7.0e6f);
@@ -2466,11 +2495,11 @@ int launch_narrow(const GemmParams& p, hipStream_t stream) {
   return MI355X_FP8_OK;
 }
 
-// the narrow-tile instantiation for a shape: one or two 32-row blocks of A, 32- or 64-column tiles
+// the narrow-tile instantiation for a shape
 int launch_narrow_for(const GemmParams& p, hipStream_t s) {
-  if (p.M > 64) return launch_narrow<2, 2>(p, s);
-  if (narrow_is_wide(p.N)) return p.M <= 32 ? launch_narrow<1, 2>(p, s) : launch_narrow<2, 2>(p, s);
-  return p.M <= 32 ? launch_narrow<1, 1>(p, s) : launch_narrow<2, 1>(p, s);
+  const NarrowForm f = narrow_form(p.M, p.N);
+  if (f.mb == 1) return f.nb == 1 ? launch_narrow<1, 1>(p, s) : launch_narrow<1, 2>(p, s);
+  return f.nb == 1 ? launch_narrow<2, 1>(p, s) : launch_narrow<2, 2>(p, s);
 }
 
 }  // namespace
