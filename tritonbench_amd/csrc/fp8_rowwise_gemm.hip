@@ -1499,12 +1499,16 @@ __global__ __launch_bounds__(kPersistWaves * 64) void gemm_skinny_persistent_ker
 //
 // Eight waves. A K step is 512 bytes: wave w of the first four fetches and multiplies the
 // step's w-th 128-byte slab of A (rows of A are L2 hits: a short queue, DA steps ahead), wave
-// 4+w fetches the same slab of the tile's 32 rows of B (from HBM, kNarrowBDist steps ahead).
+// 4+w fetches the same slab of the tile's rows of B (from HBM, DB steps ahead).
 // Loads return to a wave in order: with A and B in one queue every A line would wait behind
 // the B lines in front of it and see HBM's latency. Both go straight into LDS stages laid out
 // as [slab][row][128 bytes] with the tiled kernel's chunk swizzle; one barrier per step. The
-// four partial 32x32 (x MB) results meet in LDS at the end; wave w finishes columns 8w..8w+7
+// four partial 32x32 (x MB x NB) results meet in LDS at the end; wave w finishes columns 8w..8w+7
 // of every 32-row block.
+// What bounds it (measured with the loads taken out of the K loop: M=128, N=K=8192 13.5 instead of
+// 21.7 us; M=64, N=4096 8.2 instead of 13.0): the bytes the CUs pull from L2 together, about 17 TB/s
+// chip-wide in every form (32 KB per step and CU with 32x32 tiles, 64 KB with 64x64), not the depth of
+// either ring and not the order of LDS reads and MFMAs.
 // Workgroup g starts its walk over K at step 5g mod steps and wraps around: with a power-of-two
 // row pitch the rows in flight at one moment would otherwise agree in their low address bits
 // and crowd a few memory channels (measured, M=32, N=K=8192, K loop only: 19.8 -> 13.4 us).
@@ -1513,9 +1517,11 @@ constexpr int kNarrowKS = 512;
 // NB: 32-column blocks per tile (2: 64-column tiles, for panels of one to two 32-column tiles per CU).
 // Steps the loads run ahead of their use: what the 160 KB of LDS allow.
 constexpr int narrow_b_dist(int MB, int NB) { return NB == 1 ? 5 : MB == 1 ? 3 : 2; }
-constexpr int narrow_a_dist(int MB, int NB) { return MB == 1 && NB == 1 ? 2 : 1; }
+// A's stages: a compute wave is the only reader of the slab it fetches, so it refills a stage as soon as
+// its own fragment reads of it have returned, in the same step: as many steps ahead as there are stages.
+constexpr int narrow_a_dist(int MB, int NB) { return MB == 1 && NB == 1 ? 3 : 2; }
 constexpr size_t narrow_lds_bytes(int MB, int NB) {
-  return (size_t)(narrow_a_dist(MB, NB) + 1) * MB * 32 * kNarrowKS + (size_t)(narrow_b_dist(MB, NB) + 1) * NB * 32 * kNarrowKS;
+  return (size_t)narrow_a_dist(MB, NB) * MB * 32 * kNarrowKS + (size_t)(narrow_b_dist(MB, NB) + 1) * NB * 32 * kNarrowKS;
 }
 static_assert(narrow_lds_bytes(2, 1) <= 160 * 1024 && narrow_lds_bytes(1, 2) <= 160 * 1024 && narrow_lds_bytes(2, 2) <= 160 * 1024,
               "stage rings must fit the LDS");
@@ -1531,7 +1537,7 @@ template <int MB, int NB>
 __global__ __launch_bounds__(512) void gemm_narrow_kernel(GemmParams p) {
   constexpr int BM = 32 * MB, BN = 32 * NB, KS = kNarrowKS;
   constexpr int DA = narrow_a_dist(MB, NB), DB = narrow_b_dist(MB, NB);
-  constexpr int RA = DA + 1, RB = DB + 1;
+  constexpr int RA = DA, RB = DB + 1;
   constexpr int STA = BM * KS, STB = BN * KS;  // bytes per stage
   constexpr int LA = BM / 8, LB = BN / 8;      // wave-wide loads per wave and step (8 rows x 128 bytes each)
   static_assert((DA - 1) * LA < 64 && (DB - 1) * LB < 64, "outstanding-load counts must fit the wait instruction");
@@ -1612,40 +1618,54 @@ __global__ __launch_bounds__(512) void gemm_narrow_kernel(GemmParams p) {
 #pragma unroll
       for (int j = 0; j < 2; ++j) rd[sh][j] = l32 * kStepK + (((4 * half + 2 * sh + j) ^ swz128(l32)) * kChunk);
 
-    for (int s = 0; s < ksteps; ++s) {
-      issue_a(s + DA);
+    // The two K halves of a step are read and multiplied out of phase: while the MFMAs of one half
+    // run, the fragment reads of the next are under way (the second half of the same step, or, past
+    // the step's barrier, the first half of the next step), so neither the LDS reads nor the MFMAs
+    // of the one wave a SIMD has here wait for the other.
+    auto read_half = [&](int s, int sh, v4i (&fbh)[NB][2], v4i (&fah)[MB][2]) {
       const uint8_t* sa_rows = lds + (s % RA) * STA + wave * (BM * kStepK);
       const uint8_t* sb_rows = lds + RA * STA + (s % RB) * STB + wave * (BN * kStepK);
-      v4i fb[NB][2][2], fa[MB][2][2];
 #pragma unroll
-      for (int sh = 0; sh < 2; ++sh) {
+      for (int jb = 0; jb < NB; ++jb)
 #pragma unroll
-        for (int jb = 0; jb < NB; ++jb)
+        for (int j = 0; j < 2; ++j) fbh[jb][j] = *(const v4i*)(sb_rows + jb * 32 * kStepK + rd[sh][j]);
 #pragma unroll
-          for (int j = 0; j < 2; ++j) fb[jb][sh][j] = *(const v4i*)(sb_rows + jb * 32 * kStepK + rd[sh][j]);
+      for (int i = 0; i < MB; ++i)
 #pragma unroll
-        for (int i = 0; i < MB; ++i)
+        for (int j = 0; j < 2; ++j) fah[i][j] = *(const v4i*)(sa_rows + i * 32 * kStepK + rd[sh][j]);
+    };
+    auto mfma_half = [&](const v4i (&fbh)[NB][2], const v4i (&fah)[MB][2]) {
 #pragma unroll
-          for (int j = 0; j < 2; ++j) fa[i][sh][j] = *(const v4i*)(sa_rows + i * 32 * kStepK + rd[sh][j]);
-      }
+      for (int jb = 0; jb < NB; ++jb) {
+        const v8i vb = (v8i){fbh[jb][0][0], fbh[jb][0][1], fbh[jb][0][2], fbh[jb][0][3],
+                             fbh[jb][1][0], fbh[jb][1][1], fbh[jb][1][2], fbh[jb][1][3]};
 #pragma unroll
-      for (int sh = 0; sh < 2; ++sh) {
-#pragma unroll
-        for (int jb = 0; jb < NB; ++jb) {
-          const v8i vb = (v8i){fb[jb][sh][0][0], fb[jb][sh][0][1], fb[jb][sh][0][2], fb[jb][sh][0][3],
-                               fb[jb][sh][1][0], fb[jb][sh][1][1], fb[jb][sh][1][2], fb[jb][sh][1][3]};
-#pragma unroll
-          for (int i = 0; i < MB; ++i) {
-            const v8i va = (v8i){fa[i][sh][0][0], fa[i][sh][0][1], fa[i][sh][0][2], fa[i][sh][0][3],
-                                 fa[i][sh][1][0], fa[i][sh][1][1], fa[i][sh][1][2], fa[i][sh][1][3]};
-            acc[i][jb] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(vb, va, acc[i][jb], 0, 0, 0, 0, 0, 0);
-          }
+        for (int i = 0; i < MB; ++i) {
+          const v8i va = (v8i){fah[i][0][0], fah[i][0][1], fah[i][0][2], fah[i][0][3],
+                               fah[i][1][0], fah[i][1][1], fah[i][1][2], fah[i][1][3]};
+          acc[i][jb] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(vb, va, acc[i][jb], 0, 0, 0, 0, 0, 0);
         }
       }
+    };
+    v4i fb0[NB][2], fa0[MB][2], fb1[NB][2], fa1[MB][2];
+    read_half(0, 0, fb0, fa0);
+    for (int s = 0; s < ksteps; ++s) {
+      read_half(s, 1, fb1, fa1);
+      __builtin_amdgcn_sched_barrier(0);
+      mfma_half(fb0, fa0);
+      // every fragment of the step is in registers: this wave's slab of the A stage is free again, and
+      // the loads of step s + DA go into it (nobody else reads or writes that slab)
+      __builtin_amdgcn_sched_barrier(0);
+      __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0): the LDS reads above have returned
+      issue_a(s + DA);
       // own loads of A(s+1) have landed (the younger A(s+2) .. A(s+DA) may be in flight); past the barrier
       // everyone's have, B's included, and every wave is done reading this step's stages
       if (s + DA < ksteps) wait_loads<(DA - 1) * LA>(); else wait_loads<0>();
       __builtin_amdgcn_s_barrier();
+      if (s + 1 < ksteps) read_half(s + 1, 0, fb0, fa0);
+      __builtin_amdgcn_sched_barrier(0);
+      mfma_half(fb1, fa1);
+      __builtin_amdgcn_sched_barrier(0);
     }
 
     // ---- the four waves' partial results meet in LDS (the stages are free: last barrier passed)
