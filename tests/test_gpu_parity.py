@@ -397,6 +397,21 @@ def test_quantiser_bf16_bit_exact(gpu_device, rows, cols):
     assert torch.equal(inv.cpu().view(torch.int32), want_inv.view(torch.int32))
 
 
+@pytest.mark.parametrize("dtype,cols", [(torch.float32, 1024), (torch.float32, 1040), (torch.float32, 2048), (torch.float32, 2064),
+                                        (torch.bfloat16, 512), (torch.bfloat16, 2048), (torch.bfloat16, 2064),
+                                        (torch.bfloat16, 4096), (torch.bfloat16, 4112)])
+@pytest.mark.parametrize("rows", [1, 6, 8])
+def test_quantiser_rows_of_one_wave(gpu_device, dtype, cols, rows):
+    # rows short enough for one wave each (four per workgroup, the last workgroup partly empty), at the
+    # row lengths where the form and the chunks kept per lane change
+    x = orc.randn_f32(rows, cols, 1.0, seed=rows * 7 + cols).to(dtype)
+    want_q, want_inv = orc.fp8_row_quantize(x)
+    xq, inv = ops.fp8_row_quantize(x.to(gpu_device))
+    torch.cuda.synchronize()
+    assert torch.equal(xq.cpu().view(torch.uint8), want_q.view(torch.uint8))
+    assert torch.equal(inv.cpu().view(torch.int32), want_inv.view(torch.int32))
+
+
 def test_quantiser_rounding_at_every_code_boundary(gpu_device):
     # every finite e4m3fn value, every midpoint between neighbours (the ties) and the fp32
     # numbers just below and above each midpoint, with 448 as the row maximum so the scale is 1:

@@ -1856,19 +1856,24 @@ struct VecTraits<uint16_t> {
   }
 };
 
-template <typename SrcT, int CACHE, int THREADS>
-__global__ __launch_bounds__(THREADS) void quantize_rows_vec_kernel(const SrcT* x, uint8_t* xq,
-                                                                float* inv_scale, int K, long ldx,
-                                                                long ldq) {
+// THREADS lanes per row, ROWS rows per workgroup. Rows short enough for one wave's registers take
+// THREADS = 64 with several rows per workgroup: no LDS, no barrier, and a fraction of the workgroups
+// (short rows are bound by the rate at which workgroups start, about one per 1.2-2 ns).
+template <typename SrcT, int CACHE, int THREADS, int ROWS = 1>
+__global__ __launch_bounds__(THREADS* ROWS) void quantize_rows_vec_kernel(const SrcT* x, uint8_t* xq,
+                                                                        float* inv_scale, int K, long ldx,
+                                                                        long ldq, long rows) {
+  static_assert(ROWS == 1 || THREADS == 64, "several rows per workgroup: one wave each");
   using T = SrcTraits<SrcT>;
   using V = VecTraits<SrcT>;
   constexpr int EPV = V::EPV;
   __shared__ float wave_max[THREADS / 64];
-  const long row = blockIdx.x;
+  const long row = (long)blockIdx.x * ROWS + (ROWS > 1 ? (long)(threadIdx.x >> 6) : 0);
+  if (ROWS > 1 && row >= rows) return;  // (whole waves; this form has no barrier)
   const v4i* xr = (const v4i*)(x + row * ldx);
   uint8_t* qr = xq + row * ldq;
   const int nchunks = K / EPV;
-  const int tid = threadIdx.x;
+  const int tid = ROWS > 1 ? (int)(threadIdx.x & 63) : (int)threadIdx.x;
 
   v4i cache[CACHE];
   float amax = 0.0f;
@@ -1889,10 +1894,12 @@ __global__ __launch_bounds__(THREADS) void quantize_rows_vec_kernel(const SrcT* 
   for (int c = tid + THREADS * CACHE; c < nchunks; c += THREADS) fold(xr[c]);
 #pragma unroll
   for (int o = 32; o > 0; o >>= 1) amax = max_keep_nan(amax, __shfl_xor(amax, o));
-  if ((tid & 63) == 0) wave_max[tid >> 6] = amax;
-  __syncthreads();
+  if (THREADS > 64) {
+    if ((tid & 63) == 0) wave_max[tid >> 6] = amax;
+    __syncthreads();
 #pragma unroll
-  for (int w = 0; w < THREADS / 64; ++w) amax = max_keep_nan(amax, wave_max[w]);
+    for (int w = 0; w < THREADS / 64; ++w) amax = max_keep_nan(amax, wave_max[w]);
+  }
 
   const float scale = row_scale<SrcT>(amax);
   if (tid == 0) inv_scale[row] = T::round(1.0f / scale);
@@ -1929,8 +1936,8 @@ __global__ __launch_bounds__(THREADS) void quantize_rows_vec_kernel(const SrcT* 
   // leave as one 16-byte store per lane, BATCH runs of 1024 / BATCH contiguous bytes each.
   constexpr int BATCH = 16 / EPV;
   static_assert(CACHE % BATCH == 0, "cached rounds must split into whole batches");
-  __shared__ __attribute__((aligned(16))) uint8_t strip[THREADS / 64][1024];
-  uint8_t* mine = strip[tid >> 6];
+  __shared__ __attribute__((aligned(16))) uint8_t strip[THREADS * ROWS / 64][1024];
+  uint8_t* mine = strip[threadIdx.x >> 6];
   const int lane = tid & 63;
   constexpr int LPR = 64 / BATCH;  // lanes that store one round's bytes of this wave
 #pragma unroll
@@ -1972,25 +1979,28 @@ __global__ __launch_bounds__(THREADS) void quantize_rows_vec_kernel(const SrcT* 
 // ------------------------------------------------------------------------------------
 constexpr int kFusedRmsNorm = 0, kFusedSiluMul = 1;
 
-template <int OP, int CACHE, int THREADS>
-__global__ __launch_bounds__(THREADS) void fused_rowwise_quant_kernel(const uint16_t* x1, const uint16_t* x2,
-                                                                      float eps, uint8_t* xq, float* inv_scale,
-                                                                      int K, long ld1, long ld2, long ldq) {
+template <int OP, int CACHE, int THREADS, int ROWS = 1>
+__global__ __launch_bounds__(THREADS* ROWS) void fused_rowwise_quant_kernel(const uint16_t* x1, const uint16_t* x2,
+                                                                             float eps, uint8_t* xq, float* inv_scale,
+                                                                             int K, long ld1, long ld2, long ldq, long rows) {
+  static_assert(ROWS == 1 || THREADS == 64, "several rows per workgroup: one wave each (as in the quantiser)");
   using V = VecTraits<uint16_t>;
   constexpr int EPV = 8;
   __shared__ float wave_part[2][THREADS / 64];  // one set per reduction: neither waits for the other's readers
-  const long row = blockIdx.x;
+  const long row = (long)blockIdx.x * ROWS + (ROWS > 1 ? (long)(threadIdx.x >> 6) : 0);
+  if (ROWS > 1 && row >= rows) return;  // (whole waves; this form has no barrier)
   const v4i* r1 = (const v4i*)(x1 + row * ld1);
   // RMSNorm: the weight vector, shared by all rows; SiLU-mul: the row of the second operand
   const v4i* r2 = (const v4i*)(OP == kFusedRmsNorm ? x2 : x2 + row * ld2);
   uint8_t* qr = xq + row * ldq;
   const int nchunks = K / EPV;
-  const int tid = threadIdx.x;
+  const int tid = ROWS > 1 ? (int)(threadIdx.x & 63) : (int)threadIdx.x;
 
-  // sums (or maxima) of one value per lane over the workgroup; every lane gets the result
+  // sums (or maxima) of one value per lane over the row's lanes; every lane gets the result
   auto block_reduce = [&](int set, float v, auto op) -> float {
 #pragma unroll
     for (int o = 32; o > 0; o >>= 1) v = op(v, __shfl_xor(v, o));
+    if (THREADS == 64) return v;
     if ((tid & 63) == 0) wave_part[set][tid >> 6] = v;
     __syncthreads();
     float r = wave_part[set][0];
@@ -2087,8 +2097,8 @@ __global__ __launch_bounds__(THREADS) void fused_rowwise_quant_kernel(const uint
   };
   // pass 3: convert. Two consecutive rounds of cached chunks meet in a wave-private LDS strip and
   // leave as one 16-byte store per lane (LDS executes a wave's operations in order: no barrier).
-  __shared__ __attribute__((aligned(16))) uint8_t strip[THREADS / 64][1024];
-  uint8_t* mine = strip[tid >> 6];
+  __shared__ __attribute__((aligned(16))) uint8_t strip[THREADS * ROWS / 64][1024];
+  uint8_t* mine = strip[threadIdx.x >> 6];
   const int lane = tid & 63;
   static_assert(CACHE % 2 == 0, "cached rounds are stored in pairs");
 #pragma unroll
@@ -2773,6 +2783,16 @@ int mi355x_fp8_blockwise_gemm(const void* a, const void* b, const float* a_scale
                       : launch_tiled<128, 128, 2, 2, false, kEpiPlain, false, true>(p, s);
 }
 
+namespace {
+// Rows of at most 64 x 8 16-byte chunks are quantised by one wave each, kWaveRows rows per workgroup:
+// the number of chunks a lane keeps in registers (4 or 8), or 0 for longer rows. (Measured, bf16 rows,
+// workgroup per row -> wave per row: 16384 x 2048 quantiser 28.7 -> 19.9 us, RMSNorm form 40.8 -> 21.0,
+// SiLU-mul form 49.0 -> 27.9; 65536 x 512 75 -> 30, 132 -> 42, 170 -> 50; eight rows per workgroup
+// instead of four changed nothing.)
+constexpr int kWaveRows = 4;
+inline int row_chunks_per_lane(int64_t chunks) { return chunks <= 64 * 4 ? 4 : chunks <= 64 * 8 ? 8 : 0; }
+}  // namespace
+
 int mi355x_fp8_rowwise_quantize(const void* x, int src_type, void* xq, float* inv_scale, int64_t R,
                                 int64_t K, int64_t ldx, int64_t ldq, void* stream) {
   if (!x || !xq || !inv_scale) return fail(MI355X_FP8_EINVAL, "null pointer");
@@ -2787,15 +2807,29 @@ int mi355x_fp8_rowwise_quantize(const void* x, int src_type, void* xq, float* in
                    (reinterpret_cast<uintptr_t>(xq) & 15) == 0 && ldq % 16 == 0;
   const bool long_row = K / epv > 8 * 256;  // more chunks than 256 lanes keep in registers
   const bool short_row = K / epv <= 4 * 256;  // (bf16 source: half the registers, more workgroups per CU)
+  const int wave_cache = row_chunks_per_lane(K / epv);  // > 0: a wave per row, that many chunks per lane
+  const unsigned wave_grid = (unsigned)((R + kWaveRows - 1) / kWaveRows);
   if (vec && src_type == MI355X_FP8_SRC_F32) {
-    auto kern = long_row ? quantize_rows_vec_kernel<float, 8, 1024> : quantize_rows_vec_kernel<float, 8, 256>;
-    hipLaunchKernelGGL(kern, dim3((unsigned)R), dim3(long_row ? 1024 : 256), 0, s, (const float*)x,
-                       (uint8_t*)xq, inv_scale, (int)K, (long)ldx, (long)ldq);
+    if (wave_cache) {
+      auto kern = wave_cache == 4 ? quantize_rows_vec_kernel<float, 4, 64, kWaveRows> : quantize_rows_vec_kernel<float, 8, 64, kWaveRows>;
+      hipLaunchKernelGGL(kern, dim3(wave_grid), dim3(64 * kWaveRows), 0, s, (const float*)x, (uint8_t*)xq, inv_scale, (int)K,
+                         (long)ldx, (long)ldq, (long)R);
+    } else {
+      auto kern = long_row ? quantize_rows_vec_kernel<float, 8, 1024> : quantize_rows_vec_kernel<float, 8, 256>;
+      hipLaunchKernelGGL(kern, dim3((unsigned)R), dim3(long_row ? 1024 : 256), 0, s, (const float*)x,
+                         (uint8_t*)xq, inv_scale, (int)K, (long)ldx, (long)ldq, (long)R);
+    }
   } else if (vec && src_type == MI355X_FP8_SRC_BF16) {
-    auto kern = long_row ? quantize_rows_vec_kernel<uint16_t, 8, 1024>
-                         : short_row ? quantize_rows_vec_kernel<uint16_t, 4, 256> : quantize_rows_vec_kernel<uint16_t, 8, 256>;
-    hipLaunchKernelGGL(kern, dim3((unsigned)R), dim3(long_row ? 1024 : 256), 0, s,
-                       (const uint16_t*)x, (uint8_t*)xq, inv_scale, (int)K, (long)ldx, (long)ldq);
+    if (wave_cache) {
+      auto kern = wave_cache == 4 ? quantize_rows_vec_kernel<uint16_t, 4, 64, kWaveRows> : quantize_rows_vec_kernel<uint16_t, 8, 64, kWaveRows>;
+      hipLaunchKernelGGL(kern, dim3(wave_grid), dim3(64 * kWaveRows), 0, s, (const uint16_t*)x, (uint8_t*)xq, inv_scale, (int)K,
+                         (long)ldx, (long)ldq, (long)R);
+    } else {
+      auto kern = long_row ? quantize_rows_vec_kernel<uint16_t, 8, 1024>
+                           : short_row ? quantize_rows_vec_kernel<uint16_t, 4, 256> : quantize_rows_vec_kernel<uint16_t, 8, 256>;
+      hipLaunchKernelGGL(kern, dim3((unsigned)R), dim3(long_row ? 1024 : 256), 0, s,
+                         (const uint16_t*)x, (uint8_t*)xq, inv_scale, (int)K, (long)ldx, (long)ldq, (long)R);
+    }
   } else if (src_type == MI355X_FP8_SRC_F32) {
     hipLaunchKernelGGL(quantize_rows_kernel<float>, dim3((unsigned)R), dim3(256), 0, s, (const float*)x,
                        (uint8_t*)xq, inv_scale, (int)K, (long)ldx, (long)ldq);
@@ -2829,17 +2863,26 @@ int launch_fused_quant(int op, const void* x1, const void* x2, float eps, void* 
   const int64_t chunks = K / 8;
   const bool long_row = chunks > 8 * 256;
   const bool short_row = chunks <= 4 * 256;
-  const dim3 grid((unsigned)R), block(long_row ? 1024 : 256);
+  // > 0: a wave per row, that many chunks per lane (RMSNorm with eight chunks and their weights per lane
+  // measured behind the workgroup-per-row form: 50.1 against 47.8 us on 16384 x 4096)
+  int wave_cache = row_chunks_per_lane(chunks);
+  if (op == kFusedRmsNorm && wave_cache == 8) wave_cache = 0;
+  const dim3 grid(wave_cache ? (unsigned)((R + kWaveRows - 1) / kWaveRows) : (unsigned)R);
+  const dim3 block(wave_cache ? 64 * kWaveRows : long_row ? 1024 : 256);
   const uint16_t* a = (const uint16_t*)x1;
   const uint16_t* b = (const uint16_t*)x2;
   if (op == kFusedRmsNorm) {
-    auto kern = long_row ? fused_rowwise_quant_kernel<kFusedRmsNorm, 8, 1024>
-                         : short_row ? fused_rowwise_quant_kernel<kFusedRmsNorm, 4, 256> : fused_rowwise_quant_kernel<kFusedRmsNorm, 8, 256>;
-    hipLaunchKernelGGL(kern, grid, block, 0, s, a, b, eps, (uint8_t*)xq, inv_scale, (int)K, (long)ld1, (long)ld2, (long)ldq);
+    auto kern = wave_cache == 4 ? fused_rowwise_quant_kernel<kFusedRmsNorm, 4, 64, kWaveRows>
+                : wave_cache  ? fused_rowwise_quant_kernel<kFusedRmsNorm, 8, 64, kWaveRows>
+                : long_row    ? fused_rowwise_quant_kernel<kFusedRmsNorm, 8, 1024>
+                : short_row   ? fused_rowwise_quant_kernel<kFusedRmsNorm, 4, 256> : fused_rowwise_quant_kernel<kFusedRmsNorm, 8, 256>;
+    hipLaunchKernelGGL(kern, grid, block, 0, s, a, b, eps, (uint8_t*)xq, inv_scale, (int)K, (long)ld1, (long)ld2, (long)ldq, (long)R);
   } else {
-    auto kern = long_row ? fused_rowwise_quant_kernel<kFusedSiluMul, 8, 1024>
-                         : short_row ? fused_rowwise_quant_kernel<kFusedSiluMul, 4, 256> : fused_rowwise_quant_kernel<kFusedSiluMul, 8, 256>;
-    hipLaunchKernelGGL(kern, grid, block, 0, s, a, b, eps, (uint8_t*)xq, inv_scale, (int)K, (long)ld1, (long)ld2, (long)ldq);
+    auto kern = wave_cache == 4 ? fused_rowwise_quant_kernel<kFusedSiluMul, 4, 64, kWaveRows>
+                : wave_cache  ? fused_rowwise_quant_kernel<kFusedSiluMul, 8, 64, kWaveRows>
+                : long_row    ? fused_rowwise_quant_kernel<kFusedSiluMul, 8, 1024>
+                : short_row   ? fused_rowwise_quant_kernel<kFusedSiluMul, 4, 256> : fused_rowwise_quant_kernel<kFusedSiluMul, 8, 256>;
+    hipLaunchKernelGGL(kern, grid, block, 0, s, a, b, eps, (uint8_t*)xq, inv_scale, (int)K, (long)ld1, (long)ld2, (long)ldq, (long)R);
   }
   hipError_t e = hipGetLastError();
   if (e != hipSuccess) return fail(MI355X_FP8_ELAUNCH, "fused quantise kernel launch: %s", hipGetErrorString(e));
