@@ -398,7 +398,7 @@ def test_quantiser_bf16_bit_exact(gpu_device, rows, cols):
 
 
 @pytest.mark.parametrize("dtype,cols", [(torch.float32, 1024), (torch.float32, 1040), (torch.float32, 2048), (torch.float32, 2064),
-                                        (torch.bfloat16, 512), (torch.bfloat16, 2048), (torch.bfloat16, 2064),
+                                        (torch.bfloat16, 512), (torch.bfloat16, 1024), (torch.bfloat16, 1040), (torch.bfloat16, 2048), (torch.bfloat16, 2064),
                                         (torch.bfloat16, 4096), (torch.bfloat16, 4112)])
 @pytest.mark.parametrize("rows", [1, 6, 8])
 def test_quantiser_rows_of_one_wave(gpu_device, dtype, cols, rows):

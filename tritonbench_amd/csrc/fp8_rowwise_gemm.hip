@@ -2787,10 +2787,12 @@ namespace {
 // Rows of at most 64 x 8 16-byte chunks are quantised by one wave each, kWaveRows rows per workgroup:
 // the number of chunks a lane keeps in registers (4 or 8), or 0 for longer rows. (Measured, bf16 rows,
 // workgroup per row -> wave per row: 16384 x 2048 quantiser 28.7 -> 19.9 us, RMSNorm form 40.8 -> 21.0,
-// SiLU-mul form 49.0 -> 27.9; 65536 x 512 75 -> 30, 132 -> 42, 170 -> 50; eight rows per workgroup
+// SiLU-mul form 49.0 -> 27.9; 65536 x 512 75 -> 27, 132 -> 29, 170 -> 32; eight rows per workgroup
 // instead of four changed nothing.)
 constexpr int kWaveRows = 4;
 inline int row_chunks_per_lane(int64_t chunks) { return chunks <= 64 * 4 ? 4 : chunks <= 64 * 8 ? 8 : 0; }
+// (bf16 rows of up to 1024 elements: two rounds per lane instead of four, of which at least two would be idle)
+inline int bf16_row_chunks_per_lane(int64_t chunks) { return chunks <= 64 * 2 ? 2 : row_chunks_per_lane(chunks); }
 }  // namespace
 
 int mi355x_fp8_rowwise_quantize(const void* x, int src_type, void* xq, float* inv_scale, int64_t R,
@@ -2820,8 +2822,10 @@ int mi355x_fp8_rowwise_quantize(const void* x, int src_type, void* xq, float* in
                          (uint8_t*)xq, inv_scale, (int)K, (long)ldx, (long)ldq, (long)R);
     }
   } else if (vec && src_type == MI355X_FP8_SRC_BF16) {
-    if (wave_cache) {
-      auto kern = wave_cache == 4 ? quantize_rows_vec_kernel<uint16_t, 4, 64, kWaveRows> : quantize_rows_vec_kernel<uint16_t, 8, 64, kWaveRows>;
+    if (const int wave_cache = bf16_row_chunks_per_lane(K / epv)) {
+      auto kern = wave_cache == 2   ? quantize_rows_vec_kernel<uint16_t, 2, 64, kWaveRows>
+                  : wave_cache == 4 ? quantize_rows_vec_kernel<uint16_t, 4, 64, kWaveRows>
+                                    : quantize_rows_vec_kernel<uint16_t, 8, 64, kWaveRows>;
       hipLaunchKernelGGL(kern, dim3(wave_grid), dim3(64 * kWaveRows), 0, s, (const uint16_t*)x, (uint8_t*)xq, inv_scale, (int)K,
                          (long)ldx, (long)ldq, (long)R);
     } else {
@@ -2865,20 +2869,22 @@ int launch_fused_quant(int op, const void* x1, const void* x2, float eps, void* 
   const bool short_row = chunks <= 4 * 256;
   // > 0: a wave per row, that many chunks per lane (RMSNorm with eight chunks and their weights per lane
   // measured behind the workgroup-per-row form: 50.1 against 47.8 us on 16384 x 4096)
-  int wave_cache = row_chunks_per_lane(chunks);
+  int wave_cache = bf16_row_chunks_per_lane(chunks);
   if (op == kFusedRmsNorm && wave_cache == 8) wave_cache = 0;
   const dim3 grid(wave_cache ? (unsigned)((R + kWaveRows - 1) / kWaveRows) : (unsigned)R);
   const dim3 block(wave_cache ? 64 * kWaveRows : long_row ? 1024 : 256);
   const uint16_t* a = (const uint16_t*)x1;
   const uint16_t* b = (const uint16_t*)x2;
   if (op == kFusedRmsNorm) {
-    auto kern = wave_cache == 4 ? fused_rowwise_quant_kernel<kFusedRmsNorm, 4, 64, kWaveRows>
+    auto kern = wave_cache == 2 ? fused_rowwise_quant_kernel<kFusedRmsNorm, 2, 64, kWaveRows>
+                : wave_cache == 4 ? fused_rowwise_quant_kernel<kFusedRmsNorm, 4, 64, kWaveRows>
                 : wave_cache  ? fused_rowwise_quant_kernel<kFusedRmsNorm, 8, 64, kWaveRows>
                 : long_row    ? fused_rowwise_quant_kernel<kFusedRmsNorm, 8, 1024>
                 : short_row   ? fused_rowwise_quant_kernel<kFusedRmsNorm, 4, 256> : fused_rowwise_quant_kernel<kFusedRmsNorm, 8, 256>;
     hipLaunchKernelGGL(kern, grid, block, 0, s, a, b, eps, (uint8_t*)xq, inv_scale, (int)K, (long)ld1, (long)ld2, (long)ldq, (long)R);
   } else {
-    auto kern = wave_cache == 4 ? fused_rowwise_quant_kernel<kFusedSiluMul, 4, 64, kWaveRows>
+    auto kern = wave_cache == 2 ? fused_rowwise_quant_kernel<kFusedSiluMul, 2, 64, kWaveRows>
+                : wave_cache == 4 ? fused_rowwise_quant_kernel<kFusedSiluMul, 4, 64, kWaveRows>
                 : wave_cache  ? fused_rowwise_quant_kernel<kFusedSiluMul, 8, 64, kWaveRows>
                 : long_row    ? fused_rowwise_quant_kernel<kFusedSiluMul, 8, 1024>
                 : short_row   ? fused_rowwise_quant_kernel<kFusedSiluMul, 4, 256> : fused_rowwise_quant_kernel<kFusedSiluMul, 8, 256>;
