@@ -65,7 +65,7 @@ extern "C" {
  * number of 128-byte K steps is reduced to it.
  */
 /* Skinny family only: bit 8 pins the form with one 16-row tile of B per workgroup (the general
- * one). Without it M <= 16 with N a multiple of 16 and K one of 2048, 4096, 6144, 8192 runs
+ * one; M <= 64). Without it M <= 16 with N a multiple of 16 and K one of 2048, 4096, 6144, 8192 runs
  * the persistent form (one workgroup per CU walks a run of tiles with its share of A resident
  * in registers); every other shape runs the general form anyway. */
 #define MI355X_FP8_SKINNY_ONE_TILE      (1 << 8)

@@ -234,6 +234,15 @@ def test_shapes_the_kernel_does_not_take_are_refused(gpu_device):
             _run(gpu_device, xq, wq, xs, ws, None, _lib.VARIANT_SKINNY)
 
 
+def test_other_pins_of_the_family_stop_at_64_rows(gpu_device):
+    xq, wq, xs, ws, _ = orc.make_inputs(100, 64, 512, 1.0, False)
+    with pytest.raises(NotImplementedError):
+        _run(gpu_device, xq, wq, xs, ws, None, _lib.VARIANT_SKINNY | _lib.SKINNY_ONE_TILE)
+    want = orc.dequant_matmul(xq, wq, xs, ws, None)
+    out = _run(gpu_device, xq, wq, xs, ws, None, _lib.VARIANT_SKINNY)  # unpinned: the narrow-tile form in row blocks
+    torch.testing.assert_close(out, want, rtol=RTOL, atol=ATOL)
+
+
 def test_automatic_choice_runs_it_where_it_is_expected_to_win(gpu_device):
     # 32 x 8192 x 8192: one tile per CU, two blocks of A rows more than the persistent kernel keeps
     assert ops.select_variant(32, 8192, 8192) == _lib.VARIANT_SKINNY
