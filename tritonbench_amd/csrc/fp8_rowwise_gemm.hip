@@ -11,7 +11,7 @@
 //                            steps staged global->LDS with direct-to-LDS loads into swizzled
 //                            rings (2 or 3 stages of A, one more of B), 32x32x64 MFMA, epilogue
 //                            turned through LDS into 16-byte row stores. Tiles of 256x256,
-//                            128x128, 256x128 and 64x256; grouped and block-scaled forms.
+//                            128x128, 256x128, 64x256 and 128x256; grouped and block-scaled forms.
 //   splitk_finalize_kernel   adds the fp32 partial sums of a split-K launch, applies scales/bias.
 //   gemm_skinny_kernel       M <= 64: every workgroup owns 16 rows of B and all of K, its waves
 //                            split K between them and reduce through LDS; B is streamed once.
@@ -2168,7 +2168,7 @@ struct TileConfig {
   float stream_bytes_per_us;  // operand bytes per microsecond the configuration can stream from HBM
   float wg_stream_share;      // what one workgroup can stream, in units of 1/256 of that rate
 };
-constexpr int kNumTileConfigs = 4;
+constexpr int kNumTileConfigs = 5;
 constexpr int kNumGroupedTileConfigs = 3;  // the grouped form uses the first three
 // Measured on MI355X with normally distributed operands (clock under sustained MFMA load).
 constexpr TileConfig kTileConfigs[kNumTileConfigs] = {
@@ -2176,6 +2176,8 @@ constexpr TileConfig kTileConfigs[kNumTileConfigs] = {
     {128, 128, tiled_wgs_per_cu(128, 128), 1.00f, 0.60f, 5.0f, 4.4e6f, 1.18f},
     {256, 128, tiled_wgs_per_cu(256, 128), 0.87f, 0.87f, 5.0f, 4.0e6f, 1.1f},
     {64, 256, tiled_wgs_per_cu(64, 256), 0.75f, 0.75f, 9.0f, 5.7e6f, 1.42f},
+    // (one tile row against a wide panel: 128 x 57344 x 8192 75.2 us with 224 tiles, 128 x 28672 x 8192 58.6 us with 112)
+    {128, 256, tiled_wgs_per_cu(128, 256), 0.78f, 0.78f, 10.0f, 5.8e6f, 1.42f},
 };
 
 // The skinny kernel's run time for comparison with the tiled plans at M <= 64: a fixed part
@@ -2323,6 +2325,9 @@ inline TiledPlan plan_tiled(int64_t M, int64_t N, int64_t K, int force_config, i
       int splits, sps;
       normalise_splits(k_steps, want, splits, sps);
       if (force_splits <= 0 && splits != want) continue;  // duplicate of a smaller request
+      // (128x256 tiles are the plan for whole rows of K against wide panels; split, they measured behind what
+      // their estimate says: 128 x 8192 x 28672 66.3 us against 56.5 with 128x128 tiles)
+      if (c == 4 && force_splits <= 0 && splits > 1) continue;
       const float cost = plan_cost_us(M, N, K, c, splits, sps);
       if (best_cost < 0.0f || cost < best_cost) {
         best_cost = cost;
@@ -2647,6 +2652,7 @@ int mi355x_fp8_rowwise_gemm_ex(const void* a, const void* b, const float* a_scal
           case 1: return launch_tiled_config<128, 128, 2, 2, true>(p, s);
           case 2: return launch_tiled_config<256, 128, 2, 2, true>(p, s);
           case 3: return launch_tiled_config<64, 256, 1, 4, true>(p, s);
+          case 4: return launch_tiled_config<128, 256, 2, 2, true>(p, s);
           default: return fail(MI355X_FP8_EINVAL, "unknown tile configuration %d", plan.config);
         }
       }
