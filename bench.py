@@ -368,6 +368,9 @@ def profile_kernel(which, dev):
     elif which == "decode128_n10240":  # (more 64-column tiles than fit one round: the split-K pair of kernels)
         sets, wsp = make_sets(128, make_weights(10240, 8192, 0.02, False, dev, 8), 0.02, dev)
         fig = figures(128, 10240, 8192, False, time_steps(sets, wsp, 40, 10))
+    elif which == "decode128_n57344":  # (one tile row against the widest panel of the sweep: 128x256 tiles, all of K each)
+        sets, wsp = make_sets(128, make_weights(57344, 8192, 0.02, False, dev, 2), 0.02, dev)
+        fig = figures(128, 57344, 8192, False, time_steps(sets, wsp, 40, 10))
     elif which == "decode32":
         sets, wsp = make_sets(32, make_weights(8192, 8192, 0.02, False, dev, 8), 0.02, dev)
         fig = figures(32, 8192, 8192, False, time_steps(sets, wsp, 40, 10))
@@ -391,7 +394,7 @@ def main():
     ap.add_argument("--no-extra", action="store_true", help="headline workload only")
     ap.add_argument("--vendor", action="store_true",
                     help="also time torch._scaled_mm (hipBLASLt, row-wise scales) on every GEMM row's operands")
-    ap.add_argument("--profile-kernel", choices=["tiled", "skinny", "quantise", "fused", "grouped", "decode32", "decode128", "decode128_n10240", "ragged"],
+    ap.add_argument("--profile-kernel", choices=["tiled", "skinny", "quantise", "fused", "grouped", "decode32", "decode128", "decode128_n10240", "decode128_n57344", "ragged"],
                     help="run only that kernel's workload a few times (for rocprofv3 counter passes) and print its figures")
     args = ap.parse_args()
     global VENDOR
