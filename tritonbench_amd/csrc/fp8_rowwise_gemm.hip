@@ -2272,6 +2272,9 @@ inline float skinny_cost_us(int64_t M, int64_t N, int64_t K) {
 constexpr int kMaxSplits = 16;
 // Tile rows up to which a launch fetches B with the streaming policy (see gemm_tiled_kernel).
 constexpr int kStreamTileRows = 2;
+// (256x256 tiles: one tile row only. M=256, N=57344, K=8192 120.3 -> 109.7 us; with two tile rows, M=512, the
+// policy costs 2-3 %.)
+constexpr int stream_tile_rows(int bm, int bn) { return bm == 256 && bn == 256 ? 1 : kStreamTileRows; }
 
 struct TiledPlan {
   int config, splits, steps_per_split;
@@ -2300,12 +2303,13 @@ inline float plan_cost_us(int64_t M, int64_t N, int64_t K, int config, int split
   const long full_rounds = items / slots, rest = items % slots;
   float t = full_rounds * (sps * c.us_per_step + c.us_per_item);
   if (rest) t += sps * (rest <= kNumCu ? c.us_per_step_alone : c.us_per_step) + c.us_per_item;
-  // (one or two tile rows: B is fetched with the streaming policy, which is worth 8 %)
-  const bool streams_b = config != 0 && (M + c.bm - 1) / c.bm <= kStreamTileRows;
+  // (one or two tile rows, one for 256x256 tiles: B is fetched with the streaming policy, which is worth 8 % or more)
+  const bool streams_b = (M + c.bm - 1) / c.bm <= stream_tile_rows(c.bm, c.bn);
   // (fewer work items than CUs: the busy CUs cannot make up for the idle ones beyond their share)
   const float busy = items >= kNumCu ? 1.0f : fminf(1.0f, c.wg_stream_share * (float)items / (float)kNumCu);
   // (64x256 tiles, at most two splits: the rotated K order lifts the rate further; priced cautiously)
-  const float policy = !streams_b ? 1.0f : (config == 3 && splits <= 2) ? 1.08f * 1.1f : 1.08f;
+  // (256x256 tiles gain the most: their rate without the policy is the lowest)
+  const float policy = !streams_b ? 1.0f : (config == 3 && splits <= 2) ? 1.08f * 1.1f : config == 0 ? 1.2f : 1.08f;
   const float stream = ((float)M * (float)K + (float)N * (float)K) / (c.stream_bytes_per_us * policy * busy);
   if (t < stream) t = stream;
   if (splits > 1) t += 3.0f + 2.0f * (float)splits * (float)M * (float)N * 4.0f / 5.0e6f;
@@ -2428,7 +2432,7 @@ int launch_tiled_epilogue(const GemmParams& p, hipStream_t s) {
 template <int BM, int BN, int WAVES_M, int WAVES_N, bool MAY_STREAM>
 int launch_tiled_config(const GemmParams& p, hipStream_t s) {
   if constexpr (MAY_STREAM) {
-    if ((p.M + BM - 1) / BM <= kStreamTileRows) return launch_tiled_epilogue<BM, BN, WAVES_M, WAVES_N, true>(p, s);
+    if ((p.M + BM - 1) / BM <= stream_tile_rows(BM, BN)) return launch_tiled_epilogue<BM, BN, WAVES_M, WAVES_N, true>(p, s);
   }
   return launch_tiled_epilogue<BM, BN, WAVES_M, WAVES_N, false>(p, s);
 }
@@ -2647,8 +2651,7 @@ int mi355x_fp8_rowwise_gemm_ex(const void* a, const void* b, const float* a_scal
         p.steps_per_split = plan.steps_per_split;
         p.partial = plan.splits > 1 ? (float*)workspace : nullptr;
         switch (plan.config) {
-          // (256x256 tiles are never the plan for one or two tile rows)
-          case 0: return launch_tiled_config<256, 256, 2, 2, false>(p, s);
+          case 0: return launch_tiled_config<256, 256, 2, 2, true>(p, s);
           case 1: return launch_tiled_config<128, 128, 2, 2, true>(p, s);
           case 2: return launch_tiled_config<256, 128, 2, 2, true>(p, s);
           case 3: return launch_tiled_config<64, 256, 1, 4, true>(p, s);
