@@ -2241,7 +2241,13 @@ inline float narrow_cost_us(int64_t M, int64_t N, int64_t K) {
     return M <= 32 ? 4.0f + (float)N * (float)K / (K > 16384 ? 5.0e6f : 6.3e6f) : 8.0f + (float)N * (float)K / (K > 16384 ? 5.5e6f : 7.0e6f);
   const long tiles = (N + 31) / 32;
   const long rounds = (tiles + kNumCu - 1) / kNumCu;
-  return (float)rounds * (M <= 32 ? 3.5f + (float)K / 1024.0f * 1.38f : 4.5f + (float)K / 1024.0f * 1.62f);
+  // per 1024 bytes of K: what the CUs at work can pull from L2, or, with most of them at work and up to 32
+  // rows, what HBM delivers of B (measured at M <= 32: 8.6 us at 5120 x 5120, 8.3 at 4096 x 4096, 14.3 at 8192 x 8192)
+  const float share = fminf(1.0f, (float)tiles / (float)kNumCu);
+  const float k1024 = (float)K / 1024.0f;
+  // (with fewer than half the CUs at work the fixed part is larger than this form has it: the old rate stays)
+  if (M <= 32) return (float)rounds * (3.5f + k1024 * (tiles >= kNumCu / 2 ? fmaxf(1.08f, 1.38f * share) : 1.38f));
+  return (float)rounds * (4.5f + k1024 * (1.1f + 0.52f * share));
 }
 inline float skinny_streaming_cost_us(int64_t M, int64_t N, int64_t K) {
   // the persistent form (measured: 12.7 us at N=K=8192, 71 us at N=57344)
