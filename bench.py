@@ -540,6 +540,10 @@ def main():
         attempt("quantise_bf16_57344x8192", lambda: time_quantiser(57344, 8192, torch.bfloat16, dev, steps=20, copies=2))
         attempt("rmsnorm_quantise_bf16_8192x8192", lambda: time_fused_front_end("rmsnorm", 8192, 8192, dev))
         attempt("silu_mul_quantise_bf16_8192x8192", lambda: time_fused_front_end("silu_mul", 8192, 8192, dev))
+        # (rows of 2048 elements: the forms with a wave per row; eight sources in rotation, 0.5 GB)
+        attempt("quantise_bf16_16384x2048", lambda: time_quantiser(16384, 2048, torch.bfloat16, dev, copies=8))
+        attempt("rmsnorm_quantise_bf16_16384x2048", lambda: time_fused_front_end("rmsnorm", 16384, 2048, dev, copies=8))
+        attempt("silu_mul_quantise_bf16_16384x2048", lambda: time_fused_front_end("silu_mul", 16384, 2048, dev, copies=4))
         line["configs"] = configs
 
     if not args.no_cpu_baseline:
