@@ -2176,8 +2176,9 @@ constexpr TileConfig kTileConfigs[kNumTileConfigs] = {
     {128, 128, tiled_wgs_per_cu(128, 128), 1.00f, 0.60f, 5.0f, 4.4e6f, 1.18f},
     {256, 128, tiled_wgs_per_cu(256, 128), 0.87f, 0.87f, 5.0f, 4.0e6f, 1.1f},
     {64, 256, tiled_wgs_per_cu(64, 256), 0.75f, 0.75f, 9.0f, 5.7e6f, 1.42f},
-    // (one tile row against a wide panel: 128 x 57344 x 8192 75.2 us with 224 tiles, 128 x 28672 x 8192 58.6 us with 112)
-    {128, 256, tiled_wgs_per_cu(128, 256), 0.78f, 0.78f, 10.0f, 5.8e6f, 1.42f},
+    // (one tile row against a wide panel: 128 x 57344 x 8192 75.2 us with 224 tiles, bound by the stream rate;
+    // several tile rows: 512 x 16384 x 16384 125 us with 256 tiles, 4096 x 5120 x 13824 269 us with 640)
+    {128, 256, tiled_wgs_per_cu(128, 256), 0.90f, 0.90f, 10.0f, 5.8e6f, 1.42f},
 };
 
 // The skinny kernel's run time for comparison with the tiled plans at M <= 64: a fixed part
