@@ -21,7 +21,9 @@ SHAPES = [(32, 8192, 8192, False), (64, 8192, 8192, False), (128, 8192, 8192, Fa
           (64, 4096, 8192, False), (128, 2048, 8192, False),
           # the rest of the decode rows (M = 1, 32, 128) of the Llama-3-70B sweep
           (1, 8192, 8192, False), (1, 10240, 8192, False), (1, 57344, 8192, False), (1, 8192, 28672, False),
-          (32, 57344, 8192, False), (32, 8192, 28672, False), (128, 57344, 8192, False)]
+          (32, 57344, 8192, False), (32, 8192, 28672, False), (128, 57344, 8192, False),
+          # one tile row of 256x256 tiles with streamed B; several tile rows of the smaller configurations
+          (256, 57344, 8192, False), (512, 16384, 16384, False)]
 
 
 def _time_us(dev, m, n, k, bias, variant, sets):
