@@ -11,7 +11,7 @@
 //                            steps staged global->LDS with direct-to-LDS loads into swizzled
 //                            rings (2 or 3 stages of A, one more of B), 32x32x64 MFMA, epilogue
 //                            turned through LDS into 16-byte row stores. Tiles of 256x256,
-//                            128x128, 256x128, 64x256 and 128x256; grouped and block-scaled forms.
+//                            128x128, 256x128, 64x256, 128x256 and 192x256; grouped and block-scaled forms.
 //   splitk_finalize_kernel   adds the fp32 partial sums of a split-K launch, applies scales/bias.
 //   gemm_skinny_kernel       M <= 64: every workgroup owns 16 rows of B and all of K, its waves
 //                            split K between them and reduce through LDS; B is streamed once.
@@ -2168,7 +2168,7 @@ struct TileConfig {
   float stream_bytes_per_us;  // operand bytes per microsecond the configuration can stream from HBM
   float wg_stream_share;      // what one workgroup can stream, in units of 1/256 of that rate
 };
-constexpr int kNumTileConfigs = 5;
+constexpr int kNumTileConfigs = 6;
 constexpr int kNumGroupedTileConfigs = 3;  // the grouped form uses the first three
 // Measured on MI355X with normally distributed operands (clock under sustained MFMA load).
 constexpr TileConfig kTileConfigs[kNumTileConfigs] = {
@@ -2179,6 +2179,9 @@ constexpr TileConfig kTileConfigs[kNumTileConfigs] = {
     // (one tile row against a wide panel: 128 x 57344 x 8192 75.2 us with 224 tiles, bound by the stream rate;
     // several tile rows: 512 x 16384 x 16384 125 us with 256 tiles, 4096 x 5120 x 13824 269 us with 640)
     {128, 256, tiled_wgs_per_cu(128, 256), 0.90f, 0.90f, 10.0f, 5.8e6f, 1.42f},
+    // (panels whose 256-column tiles come to more than half a round with 256 rows each but fit one with 192:
+    // 1024 x 10240 x 8192 73.3 us with 240 tiles, 2048 x 10240 x 8192 135.4 us with 440)
+    {192, 256, tiled_wgs_per_cu(192, 256), 1.00f, 1.00f, 9.0f, 4.0e6f, 1.42f},
 };
 
 // The skinny kernel's run time for comparison with the tiled plans at M <= 64: a fixed part
@@ -2338,7 +2341,7 @@ inline TiledPlan plan_tiled(int64_t M, int64_t N, int64_t K, int force_config, i
       if (force_splits <= 0 && splits != want) continue;  // duplicate of a smaller request
       // (128x256 tiles are the plan for whole rows of K against wide panels; split, they measured behind what
       // their estimate says: 128 x 8192 x 28672 66.3 us against 56.5 with 128x128 tiles)
-      if (c == 4 && force_splits <= 0 && splits > 1) continue;
+      if (c >= 4 && force_splits <= 0 && splits > 1) continue;  // (192x256 tiles were not measured split either)
       const float cost = plan_cost_us(M, N, K, c, splits, sps);
       if (best_cost < 0.0f || cost < best_cost) {
         best_cost = cost;
@@ -2663,6 +2666,7 @@ int mi355x_fp8_rowwise_gemm_ex(const void* a, const void* b, const float* a_scal
           case 2: return launch_tiled_config<256, 128, 2, 2, true>(p, s);
           case 3: return launch_tiled_config<64, 256, 1, 4, true>(p, s);
           case 4: return launch_tiled_config<128, 256, 2, 2, true>(p, s);
+          case 5: return launch_tiled_config<192, 256, 2, 2, true>(p, s);
           default: return fail(MI355X_FP8_EINVAL, "unknown tile configuration %d", plan.config);
         }
       }
