@@ -2181,7 +2181,8 @@ constexpr TileConfig kTileConfigs[kNumTileConfigs] = {
     {128, 256, tiled_wgs_per_cu(128, 256), 0.90f, 0.90f, 10.0f, 5.8e6f, 1.42f},
     // (panels whose 256-column tiles come to more than half a round with 256 rows each but fit one with 192:
     // 1024 x 10240 x 8192 73.3 us with 240 tiles, 2048 x 10240 x 8192 135.4 us with 440)
-    {192, 256, tiled_wgs_per_cu(192, 256), 1.00f, 1.00f, 9.0f, 4.0e6f, 1.42f},
+    // (one tile row against a wide panel: 192 x 57344 x 8192 89.2 us)
+    {192, 256, tiled_wgs_per_cu(192, 256), 1.00f, 1.00f, 9.0f, 4.9e6f, 1.42f},
 };
 
 // The skinny kernel's run time for comparison with the tiled plans at M <= 64: a fixed part
@@ -2317,10 +2318,16 @@ inline float plan_cost_us(int64_t M, int64_t N, int64_t K, int config, int split
   const bool streams_b = (M + c.bm - 1) / c.bm <= stream_tile_rows(c.bm, c.bn);
   // (fewer work items than CUs: the busy CUs cannot make up for the idle ones beyond their share)
   const float busy = items >= kNumCu ? 1.0f : fminf(1.0f, c.wg_stream_share * (float)items / (float)kNumCu);
-  // (64x256 tiles, at most two splits: the rotated K order lifts the rate further; priced cautiously)
+  // (64x256 tiles, unsplit: the rotated K order lifts the rate further; with two splits the plan measured at the
+  // plain rate, 48 x 28672 x 8192 47.5 us)
   // (256x256 tiles gain the most: their rate without the policy is the lowest)
-  const float policy = !streams_b ? 1.0f : (config == 3 && splits <= 2) ? 1.08f * 1.1f : config == 0 ? 1.2f : 1.08f;
-  const float stream = ((float)M * (float)K + (float)N * (float)K) / (c.stream_bytes_per_us * policy * busy);
+  const float policy = !streams_b ? 1.0f : (config == 3 && splits == 1) ? 1.08f * 1.1f : config == 0 ? 1.2f : 1.08f;
+  // (128x128 tiles: the rate was measured with full tiles; rows of a tile past M are not fetched, and what a CU
+  // has to take in beside its rows of B shrinks with them: 64 x 28672 x 8192 unsplit 42.4 us = 6.3 MB/us)
+  const float rows_a = (float)M / (float)((M + c.bm - 1) / c.bm);
+  // (not below 33 rows: there the estimate would undercut the streaming kernels, which measure 25 % ahead)
+  const float fill = config == 1 && M > 32 ? fmaxf(0.75f, (rows_a + (float)c.bn) / (float)(c.bm + c.bn)) : 1.0f;
+  const float stream = ((float)M * (float)K + (float)N * (float)K) * fill / (c.stream_bytes_per_us * policy * busy);
   if (t < stream) t = stream;
   if (splits > 1) t += 3.0f + 2.0f * (float)splits * (float)M * (float)N * 4.0f / 5.0e6f;
   return t;
