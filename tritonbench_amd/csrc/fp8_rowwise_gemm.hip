@@ -2264,10 +2264,15 @@ inline float skinny_streaming_cost_us(int64_t M, int64_t N, int64_t K) {
   float r = M <= 8 ? 7.2e6f : rate[b];  // (a few rows of A: its loads hit in L1 almost always)
   // two blocks, one round of workgroups (two per CU) and a short K: everything is in flight at once
   if (b == 1 && N <= 16 * 2 * kNumCu && K <= 8192) r = 4.9e6f;
-  if (b >= 2) {
+  // The kernel takes as long as its busiest CU: workgroups are dealt out in rounds of one per CU, and a last
+  // round that reaches only some CUs costs a whole one (16 x 5120 x 13824: 20.8 us with 320 workgroups, where
+  // 4096 x 14336 with 256 takes 12.9).
+  // (With one or two blocks of A a single round that leaves CUs idle is left as it was: those shapes are a few
+  // microseconds long and bound by the launch, 32 x 2048 x 2048 4.5 us.)
+  {
     const long wgs = (N + (b == 3 ? 31 : 15)) / (b == 3 ? 32 : 16);
     const long rounds = (wgs + kNumCu - 1) / kNumCu;
-    r *= (float)wgs / (float)(rounds * kNumCu);
+    if (b >= 2 || rounds > 1) r *= (float)wgs / (float)(rounds * kNumCu);
   }
   return 5.0f + (float)N * (float)K / r;
 }
