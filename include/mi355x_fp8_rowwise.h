@@ -19,8 +19,10 @@
  *   - fp8 is OCP e4m3fn (bias 7, max 448, no inf, NaN = 0x7f/0xff), one byte per element;
  *   - bf16 is the upper 16 bits of an IEEE binary32, rounded to nearest even;
  *   - `stream` is a hipStream_t passed as void* (NULL = the null stream);
- *   - calls only ENQUEUE work: no allocation, no host synchronisation, so they may be
- *     recorded into a HIP graph;
+ *   - after mi355x_fp8_rowwise_init() on the device, calls only ENQUEUE work: no allocation, no
+ *     host synchronisation, no attribute or query call, so they may be recorded into a HIP graph;
+ *     state kept on the host is per device, written with atomics, and the same whichever thread
+ *     wrote it (the library is re-entrant per stream);
  *   - the library borrows all pointers for the duration of the enqueued work and owns
  *     no device memory.
  *
@@ -39,7 +41,7 @@
 extern "C" {
 #endif
 
-#define MI355X_FP8_ABI_VERSION 1
+#define MI355X_FP8_ABI_VERSION 2
 
 #define MI355X_FP8_OK        0
 #define MI355X_FP8_EINVAL   (-1)
@@ -85,6 +87,19 @@ extern "C" {
 #define MI355X_FP8_SRC_BF16  1
 
 int mi355x_fp8_rowwise_abi_version(void);
+
+/*
+ * Sets the CURRENT HIP device up for this library: checks that it is the part the kernels are
+ * scheduled for (256 compute units), raises the dynamic-LDS limit of every kernel on it and looks
+ * up the address of the built-in scratch buffer. It has no counterpart in the reference (PyTorch
+ * initialises its own libraries on first use). These are the only HIP calls of the library that
+ * are not enqueues; after a successful init on a device every entry point below only launches
+ * kernels there, whatever shape, variant or instantiation a call is the first to use, so a call
+ * may be recorded into a HIP graph without an eager call of the same kind before it. Idempotent
+ * and thread-safe; call it once per device, outside graph capture. An entry point called on a
+ * device that was never initialised does the same set-up on the way (not under capture, then).
+ */
+int mi355x_fp8_rowwise_init(void);
 
 const char* mi355x_fp8_rowwise_last_error(void);
 
@@ -146,11 +161,14 @@ int mi355x_fp8_rowwise_gemm_ex(const void* a, const void* b,
  * buffer of MI355X_FP8_NOALLOC_SCRATCH_BYTES built into the library's device code (one copy per
  * GPU, held until the process ends). The call allocates and frees nothing.
  *
- * A plan that needs more than the buffer holds is refused with MI355X_FP8_ENOTSUP (use the
- * workspace form for it); plans that need no workspace run at any size. All calls on one GPU
+ * When the plan the library would choose needs more than the buffer holds, the call runs the
+ * cheapest plan whose partial sums fit (as the workspace form does with a workspace that is too
+ * small); only a call that names a split-K factor the buffer cannot hold is refused with
+ * MI355X_FP8_ENOTSUP (use the workspace form for it). All calls on one GPU
  * share that GPU's buffer: calls that may overlap there (different streams, concurrently
- * replayed graphs) race on it and must be ordered by the caller. The first call on a device
- * looks the buffer's address up; make that call outside graph capture.
+ * replayed graphs) race on it and must be ordered by the caller. The buffer's address is looked
+ * up by mi355x_fp8_rowwise_init() (or by the first call on a device that was not initialised:
+ * make that call outside graph capture).
  */
 #define MI355X_FP8_NOALLOC_SCRATCH_BYTES (64u << 20)
 int mi355x_fp8_rowwise_gemm_noalloc(const void* a, const void* b,

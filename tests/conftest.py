@@ -10,6 +10,7 @@ if ROOT not in sys.path:
 
 def pytest_configure(config):
     config.addinivalue_line("markers", "gpu: needs a ROCm GPU (MI355X); run with -m gpu")
+    config.addinivalue_line("markers", "perf: asserts on measured run times (calibration of the dispatch), not on results")
 
 
 @pytest.fixture(scope="session")

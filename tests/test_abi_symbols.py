@@ -133,3 +133,14 @@ def test_leading_dimension_limits_are_checked_on_the_host():
     assert call(16, 16, limit_c + 1) == _lib.ENOTSUP and "leading dimension too large" in _lib.last_error()
     # smaller than the row is a different complaint
     assert call(8, 16, 16) == _lib.EINVAL and "smaller than the row" in _lib.last_error()
+
+
+def test_init_reports_a_missing_device_instead_of_crashing():
+    import pytest
+    import torch
+
+    if torch.cuda.is_available():
+        pytest.skip("a device is visible: the set-up itself is exercised by the gpu tests")
+    lib = _lib.load()
+    assert lib.mi355x_fp8_rowwise_init() == _lib.ELAUNCH
+    assert "hipGetDevice" in _lib.last_error()

@@ -5,13 +5,17 @@ clearly slower than one of its alternatives. Needs an MI355X.
 
 Timing: a captured graph of 16 launches over 4 rotating operand sets (cold weights, as a model's
 are), best of 4 replays after a warm-up replay. The bar is 12 %: the spread of repeated
-measurements of one plan on these shapes is 2-4 %."""
+measurements of one plan on these shapes is 2-4 %.
+
+These are wall-clock assertions, not parity: they carry the `perf` marker beside `gpu`
+(`-m "gpu and not perf"` leaves them out), every shape prints its margin, and the file sorts behind
+every parity file so that a noisy replay cannot keep `pytest -x` from reaching those."""
 import pytest
 import torch
 
 from tritonbench_amd import _lib, ops
 
-pytestmark = pytest.mark.gpu
+pytestmark = [pytest.mark.gpu, pytest.mark.perf]
 
 TOLERANCE = 1.12
 # decode- and small-prefill-sized rows of the Llama-3-70B projection sweep, and the small ragged shape with bias
@@ -90,6 +94,7 @@ def test_automatic_choice_is_close_to_the_best_alternative(gpu_device, m, n, k, 
         if rnd >= 1 and auto <= TOLERANCE * min(times.values()):
             break
     best_name = min(times, key=times.get)
-    print(f"  automatic {auto:.1f} us; " + ", ".join(f"{nm} {t:.1f}" for nm, t in times.items()), flush=True)
+    print(f"  automatic {auto:.1f} us = {auto / times[best_name]:.3f} x best ('{best_name}' {times[best_name]:.1f} us; "
+          f"bar {TOLERANCE:.2f}); " + ", ".join(f"{nm} {t:.1f}" for nm, t in times.items()), flush=True)
     assert auto <= TOLERANCE * times[best_name], (
         f"automatic choice takes {auto:.1f} us, '{best_name}' {times[best_name]:.1f} us: the cost tables need recalibrating")

@@ -70,14 +70,20 @@ def test_no_alloc_entry_matches_the_workspace_entry(gpu_device):
     assert cases[2][-1] == 0
     assert cases[1][-1] < cases[0][-1]
 
-    # every output tensor exists by now: between here and the comparison nothing is allocated
+    # Every output tensor exists by now, and the device was set up (scratch address looked up) when the
+    # operands above were made: between here and the comparison nothing is allocated, by PyTorch
+    # (its own counter) or by anybody else in the process (the driver's free-memory figure sees a
+    # hipMalloc inside the library too).
     torch.cuda.synchronize()
     before = torch.cuda.memory_allocated(gpu_device)
+    free_before, _ = torch.cuda.mem_get_info(gpu_device)
     for (m, n, k, bias, xq, wq, xs, ws, b, host, want, got, need) in cases:
         print(f"no-alloc entry {m}x{n}x{k} bias={bias} scratch bytes {need}", flush=True)
         _no_alloc(lib, xq, wq, xs, ws, b, got, variant)
     torch.cuda.synchronize()
+    free_after, _ = torch.cuda.mem_get_info(gpu_device)
     assert torch.cuda.memory_allocated(gpu_device) == before
+    assert free_after >= free_before, f"device memory shrank by {free_before - free_after} bytes across the calls"
 
     for (m, n, k, bias, xq, wq, xs, ws, b, host, want, got, need) in cases:
         assert np.array_equal(_bits(got), _bits(want)), f"{m}x{n}x{k}: differs from the workspace entry point"
@@ -97,8 +103,40 @@ def test_no_alloc_entry_matches_the_workspace_entry(gpu_device):
     assert np.array_equal(_bits(got), _bits(want))
 
 
+@pytest.mark.gpu
+def test_no_alloc_entry_runs_a_smaller_plan_when_the_automatic_one_does_not_fit(gpu_device):
+    """An automatic plan that wants more scratch than the buffer holds is not an error: the call
+    runs the cheapest plan that fits, exactly as the workspace entry point does with a workspace of
+    the buffer's size (bit-identical), and agrees with the full-workspace plan to the tolerance."""
+    from tritonbench_amd import ops
+
+    lib = _lib.load()
+    m, n, k = 768, 8192, 65536
+    need = lib.mi355x_fp8_rowwise_workspace_bytes(m, n, k, _lib.VARIANT_AUTO)
+    assert need > _lib.NOALLOC_SCRATCH_BYTES, "the shape is meant to want more scratch than the buffer holds"
+    g = torch.Generator(device=gpu_device)
+    g.manual_seed(99)
+    xq, xs = ops.fp8_row_quantize(torch.randn((m, k), generator=g, device=gpu_device))
+    wq, ws = ops.fp8_row_quantize(torch.randn((n, k), generator=g, device=gpu_device))
+    full = torch.empty((m, n), dtype=torch.bfloat16, device=gpu_device)
+    _with_workspace(lib, xq, wq, xs, ws, None, full, _lib.VARIANT_AUTO)
+    same_size = torch.empty_like(full)
+    space = torch.empty(_lib.NOALLOC_SCRATCH_BYTES, dtype=torch.uint8, device=gpu_device)
+    st = lib.mi355x_fp8_rowwise_gemm(_ptr(xq), _ptr(wq), _ptr(xs), _ptr(ws), None, _ptr(same_size), m, n, k, k, k, n,
+                                     space.data_ptr(), _lib.NOALLOC_SCRATCH_BYTES, _lib.VARIANT_AUTO,
+                                     torch.cuda.current_stream().cuda_stream)
+    _lib.check(st, "mi355x_fp8_rowwise_gemm")
+    got = torch.full_like(full, float("nan"))
+    print(f"no-alloc entry {m}x{n}x{k}: automatic plan wants {need} bytes", flush=True)
+    _no_alloc(lib, xq, wq, xs, ws, None, got, _lib.VARIANT_AUTO)
+    torch.cuda.synchronize()
+    assert np.array_equal(_bits(got), _bits(same_size))
+    torch.testing.assert_close(got, full, rtol=1e-2, atol=1e-2)
+
+
 def test_no_alloc_entry_refuses_plans_beyond_its_buffer():
-    """Host arithmetic only: the request is turned away before any device call."""
+    """Host arithmetic only: a split factor the caller named and the buffer cannot hold is turned
+    away before any device call."""
     lib = _lib.load()
     m = n = 2048
     k = 4096

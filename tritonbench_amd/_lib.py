@@ -11,7 +11,7 @@ from ctypes import c_char_p, c_int, c_int64, c_size_t, c_void_p
 
 from .build import LIB_PATH
 
-ABI_VERSION = 1
+ABI_VERSION = 2
 
 OK = 0
 EINVAL = -1
@@ -56,6 +56,7 @@ SRC_BF16 = 1
 # symbol -> (restype, argtypes); must list every function the header declares
 SIGNATURES = {
     "mi355x_fp8_rowwise_abi_version": (c_int, []),
+    "mi355x_fp8_rowwise_init": (c_int, []),
     "mi355x_fp8_rowwise_last_error": (c_char_p, []),
     "mi355x_fp8_rowwise_select_variant": (c_int, [c_int64, c_int64, c_int64]),
     "mi355x_fp8_rowwise_workspace_bytes": (c_size_t, [c_int64, c_int64, c_int64, c_int]),
@@ -142,6 +143,22 @@ def load() -> ctypes.CDLL:
             raise RuntimeError(f"{LIB_PATH}: ABI version {got}, this binding expects {ABI_VERSION}")
         _lib = lib
     return _lib
+
+
+_initialised = set()
+
+
+def init_device(index: int) -> None:
+    """Sets device `index` up for the library (mi355x_fp8_rowwise_init: device check, LDS limits of
+    every kernel, scratch address), once per process and device. After it every entry point only
+    enqueues work there, so any call may be the first of its kind under graph capture."""
+    if index in _initialised:
+        return
+    import torch
+
+    with torch.cuda.device(index):
+        check(load().mi355x_fp8_rowwise_init(), "mi355x_fp8_rowwise_init")
+    _initialised.add(index)
 
 
 def last_error() -> str:

@@ -2372,39 +2372,59 @@ inline TiledPlan plan_from_variant(int64_t M, int64_t N, int64_t K, int variant,
   return plan_tiled(M, N, K, cfg, spl, spl > 0 ? spl : max_splits);
 }
 
-// Raises a kernel's dynamic-LDS limit once per device (the attribute belongs to the device's
-// copy of the code object). Idempotent, so a race between threads is harmless.
 constexpr int kMaxDevices = 64;
 // The tile walk, the grid sizes and the cost tables are written for the whole part: 256 CUs in 8
 // XCDs. A device that reports another CU count (a partitioned mode, another product) would be
-// scheduled wrongly without any error, so it is turned away here, once per device.
+// scheduled wrongly without any error, so it is turned away, once per device, when the device is
+// set up.
 int check_device_shape(int dev) {
-  static std::atomic<int> seen[kMaxDevices];  // 0 unknown, 1 fits, -1 does not
-  const bool tracked = dev >= 0 && dev < kMaxDevices;
-  int state = tracked ? seen[dev].load(std::memory_order_relaxed) : 0;
   int cus = 0;
-  if (state == 0) {
-    const hipError_t e = hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev);
-    if (e != hipSuccess) return fail(MI355X_FP8_ELAUNCH, "hipDeviceGetAttribute: %s", hipGetErrorString(e));
-    state = cus == kNumCu ? 1 : -1;
-    if (tracked) seen[dev].store(state, std::memory_order_relaxed);
-  }
-  if (state < 0)
+  const hipError_t e = hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev);
+  if (e != hipSuccess) return fail(MI355X_FP8_ELAUNCH, "hipDeviceGetAttribute: %s", hipGetErrorString(e));
+  if (cus != kNumCu)
     return fail(MI355X_FP8_ENOTSUP, "device %d does not report the %d compute units these kernels are scheduled for "
                 "(a partitioned mode or another part)", dev, kNumCu);
   return MI355X_FP8_OK;
 }
 
-int raise_lds_limit(const void* kernel, size_t lds_bytes, bool (&done)[kMaxDevices]) {
+// Every kernel instantiation that needs more dynamic LDS than the default limit enters itself in
+// this table while the library is loaded (static initialisation, before any call can arrive).
+// Setting a device up walks the table once and raises each kernel's limit there, so that no
+// launch path has anything but the launch itself to do: a caller whose first use of some
+// instantiation happens under graph capture meets no attribute call.
+struct LdsKernel {
+  const void* kernel;
+  size_t lds_bytes;
+};
+constexpr int kMaxLdsKernels = 256;
+LdsKernel g_lds_kernels[kMaxLdsKernels];
+int g_num_lds_kernels = 0;
+bool g_lds_table_overflow = false;
+bool register_lds_kernel(const void* kernel, size_t lds_bytes) {
+  if (g_num_lds_kernels < kMaxLdsKernels) g_lds_kernels[g_num_lds_kernels++] = {kernel, lds_bytes};
+  else g_lds_table_overflow = true;
+  return true;
+}
+template <auto Kernel, size_t LdsBytes>
+struct LdsLimit {
+  static inline const bool registered = register_lds_kernel(reinterpret_cast<const void*>(Kernel), LdsBytes);
+};
+
+// 0 = not set up, 1 = ready, -1 = refused (wrong device shape). Setting a device up twice from two
+// threads is harmless: every step is idempotent.
+std::atomic<int> g_device_state[kMaxDevices];
+std::atomic<void*> g_scratch_ptr[kMaxDevices];
+int setup_device(int dev);
+
+// The current device, set up. The only HIP call on the ready path is hipGetDevice.
+int ready_device(int* dev_out = nullptr) {
   int dev = 0;
-  hipError_t e = hipGetDevice(&dev);
+  const hipError_t e = hipGetDevice(&dev);
   if (e != hipSuccess) return fail(MI355X_FP8_ELAUNCH, "hipGetDevice: %s", hipGetErrorString(e));
-  if (dev >= 0 && dev < kMaxDevices && done[dev]) return MI355X_FP8_OK;
-  if (const int st = check_device_shape(dev)) return st;
-  e = hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
-  if (e != hipSuccess) return fail(MI355X_FP8_ELAUNCH, "hipFuncSetAttribute: %s", hipGetErrorString(e));
-  if (dev >= 0 && dev < kMaxDevices) done[dev] = true;
-  return MI355X_FP8_OK;
+  if (dev < 0 || dev >= kMaxDevices) return fail(MI355X_FP8_ENOTSUP, "device index %d beyond %d", dev, kMaxDevices - 1);
+  if (dev_out) *dev_out = dev;
+  if (g_device_state[dev].load(std::memory_order_acquire) == 1) return MI355X_FP8_OK;
+  return setup_device(dev);
 }
 
 template <int BM, int BN, int WAVES_M, int WAVES_N, bool KTAIL, int EPI, bool GROUPED = false, bool BLOCKSCALE = false,
@@ -2419,9 +2439,9 @@ int launch_tiled(GemmParams p, hipStream_t stream) {
   const long total = (long)p.tiles_m * p.tiles_n * p.splits;
   const long slots = (long)kNumCu * tiled_wgs_per_cu(BM, BN, BLOCKSCALE, DIST);
   long grid = total < slots ? ((total + kNumXcd - 1) / kNumXcd) * kNumXcd : slots;
-  auto kern = gemm_tiled_kernel<BM, BN, WAVES_M, WAVES_N, KTAIL, EPI, GROUPED, BLOCKSCALE, DIST, STREAM_B>;
-  static bool attr_done[kMaxDevices] = {};
-  if (const int st = raise_lds_limit((const void*)kern, lds_bytes, attr_done)) return st;
+  constexpr auto kern = gemm_tiled_kernel<BM, BN, WAVES_M, WAVES_N, KTAIL, EPI, GROUPED, BLOCKSCALE, DIST, STREAM_B>;
+  (void)LdsLimit<kern, lds_bytes>::registered;
+  if (const int st = ready_device()) return st;
   hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(threads), lds_bytes, stream, p);
   hipError_t e = hipGetLastError();
   if (e != hipSuccess) return fail(MI355X_FP8_ELAUNCH, "tiled kernel launch: %s", hipGetErrorString(e));
@@ -2463,9 +2483,9 @@ template <int MT, int NTW, int DEPTH, int KW>
 int launch_skinny(const GemmParams& p, hipStream_t stream) {
   constexpr size_t lds_bytes = (size_t)KW * (NTW + MT) * 16 * kStepK;
   static_assert(lds_bytes <= 160 * 1024, "transpose buffers must fit the 160 KB LDS");
-  auto kern = gemm_skinny_kernel<MT, NTW, DEPTH, KW>;
-  static bool attr_done[kMaxDevices] = {};
-  if (const int st = raise_lds_limit((const void*)kern, lds_bytes, attr_done)) return st;
+  constexpr auto kern = gemm_skinny_kernel<MT, NTW, DEPTH, KW>;
+  (void)LdsLimit<kern, lds_bytes>::registered;
+  if (const int st = ready_device()) return st;
   const unsigned grid = (unsigned)((p.N + 16 * NTW - 1) / (16 * NTW));
   hipLaunchKernelGGL(kern, dim3(grid), dim3(KW * 64), lds_bytes, stream, p);
   hipError_t e = hipGetLastError();
@@ -2477,26 +2497,42 @@ int launch_skinny(const GemmParams& p, hipStream_t stream) {
 // Split-K plans park their fp32 partial sums in device memory between the two launches. Callers
 // that cannot bring a workspace (HIP graph capture, serving loops that may not allocate) get this
 // array instead: every device the library is loaded on holds its own copy until the process
-// ends. In host code the array's name is only a handle for the symbol look-up below; kernels,
-// fills and copies take the per-device address that look-up returns.
+// ends. In host code the array's name is only a handle for the symbol look-up in setup_device();
+// kernels, fills and copies take the per-device address that look-up returns.
 constexpr size_t kScratchBytes = (size_t)MI355X_FP8_NOALLOC_SCRATCH_BYTES;
 static __device__ __align__(256) unsigned char scratch[kScratchBytes];
-std::atomic<void*> g_scratch_ptr[kMaxDevices];
 
-// Address of the current device's copy of `scratch` (looked up once per device).
+// Sets the current device `dev` up: checks its shape, raises the dynamic-LDS limit of every
+// registered kernel on it and looks up the address of its copy of `scratch`. None of this is an
+// enqueue, so it belongs in front of any graph capture: mi355x_fp8_rowwise_init() does it by name,
+// and a first call on a device that was never initialised does it on the way.
+int setup_device(int dev) {
+  if (g_device_state[dev].load(std::memory_order_acquire) < 0)
+    return fail(MI355X_FP8_ENOTSUP, "device %d does not report the %d compute units these kernels are scheduled for "
+                "(a partitioned mode or another part)", dev, kNumCu);
+  if (g_lds_table_overflow) return fail(MI355X_FP8_ELAUNCH, "kernel table overflow (more than %d instantiations)", kMaxLdsKernels);
+  if (const int st = check_device_shape(dev)) {
+    if (st == MI355X_FP8_ENOTSUP) g_device_state[dev].store(-1, std::memory_order_release);
+    return st;
+  }
+  for (int i = 0; i < g_num_lds_kernels; ++i) {
+    const hipError_t e = hipFuncSetAttribute(g_lds_kernels[i].kernel, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                             (int)g_lds_kernels[i].lds_bytes);
+    if (e != hipSuccess) return fail(MI355X_FP8_ELAUNCH, "hipFuncSetAttribute: %s", hipGetErrorString(e));
+  }
+  void* ptr = nullptr;
+  const hipError_t e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+  if (e != hipSuccess || !ptr) return fail(MI355X_FP8_ELAUNCH, "hipGetSymbolAddress(scratch): %s", hipGetErrorString(e));
+  g_scratch_ptr[dev].store(ptr, std::memory_order_release);  // every thread finds the same address
+  g_device_state[dev].store(1, std::memory_order_release);
+  return MI355X_FP8_OK;
+}
+
+// Address of the current device's copy of `scratch`.
 int scratch_of_current_device(void** out) {
   int dev = 0;
-  hipError_t e = hipGetDevice(&dev);
-  if (e != hipSuccess) return fail(MI355X_FP8_ELAUNCH, "hipGetDevice: %s", hipGetErrorString(e));
-  if (dev < 0 || dev >= kMaxDevices) return fail(MI355X_FP8_ENOTSUP, "device index %d beyond %d", dev, kMaxDevices - 1);
-  void* ptr = g_scratch_ptr[dev].load(std::memory_order_acquire);
-  if (!ptr) {
-    e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
-    if (e != hipSuccess || !ptr)
-      return fail(MI355X_FP8_ELAUNCH, "hipGetSymbolAddress(scratch): %s", hipGetErrorString(e));
-    g_scratch_ptr[dev].store(ptr, std::memory_order_release);  // every thread finds the same address
-  }
-  *out = ptr;
+  if (const int st = ready_device(&dev)) return st;
+  *out = g_scratch_ptr[dev].load(std::memory_order_acquire);
   return MI355X_FP8_OK;
 }
 
@@ -2514,9 +2550,9 @@ inline bool persistent_skinny_fits(int64_t M, int64_t N, int64_t K) {
 template <int SPW, int MT, int LAG, bool VEC>
 int launch_skinny_persistent(const GemmParams& p, hipStream_t stream) {
   constexpr size_t lds_bytes = persistent_lds_bytes(MT);
-  auto kern = gemm_skinny_persistent_kernel<SPW, MT, LAG, VEC>;
-  static bool attr_done[kMaxDevices] = {};
-  if (const int st = raise_lds_limit((const void*)kern, lds_bytes, attr_done)) return st;
+  constexpr auto kern = gemm_skinny_persistent_kernel<SPW, MT, LAG, VEC>;
+  (void)LdsLimit<kern, lds_bytes>::registered;
+  if (const int st = ready_device()) return st;
   const long ntiles = p.N / 16;
   const unsigned grid = (unsigned)(ntiles < kNumCu ? ntiles : kNumCu);
   GemmParams q = p;
@@ -2543,9 +2579,9 @@ int launch_skinny_persistent_steps(const GemmParams& p, hipStream_t s) {
 template <int MB, int NB>
 int launch_narrow(const GemmParams& p, hipStream_t stream) {
   constexpr size_t lds_bytes = narrow_lds_bytes(MB, NB);
-  auto kern = gemm_narrow_kernel<MB, NB>;
-  static bool attr_done[kMaxDevices] = {};
-  if (const int st = raise_lds_limit((const void*)kern, lds_bytes, attr_done)) return st;
+  constexpr auto kern = gemm_narrow_kernel<MB, NB>;
+  (void)LdsLimit<kern, lds_bytes>::registered;
+  if (const int st = ready_device()) return st;
   const unsigned tiles = (unsigned)((p.N + 32 * NB - 1) / (32 * NB));
   const unsigned row_blocks = (unsigned)((p.M + 32 * MB - 1) / (32 * MB));
   // (with row blocks the kernel deals tiles out per XCD: whole rounds of the XCDs)
@@ -2568,6 +2604,8 @@ int launch_narrow_for(const GemmParams& p, hipStream_t s) {
 extern "C" {
 
 int mi355x_fp8_rowwise_abi_version(void) { return MI355X_FP8_ABI_VERSION; }
+
+int mi355x_fp8_rowwise_init(void) { return ready_device(); }
 
 const char* mi355x_fp8_rowwise_last_error(void) { return g_err; }
 
@@ -2663,7 +2701,10 @@ int mi355x_fp8_rowwise_gemm_ex(const void* a, const void* b, const float* a_scal
           if ((plan_bits >> 16) & 0xff)
             return fail(MI355X_FP8_EINVAL, "split-K factor %d needs %zu bytes of workspace (got %zu)",
                         plan.splits, need, workspace ? workspace_bytes : (size_t)0);
-          plan = plan_from_variant(M, N, K, plan_bits, 1);
+          // the cheapest plan whose partial planes fit what the caller brought (none: the unsplit plans)
+          const size_t plane = (size_t)M * (size_t)N * sizeof(float);
+          const size_t fit = workspace ? workspace_bytes / plane : 0;
+          plan = plan_from_variant(M, N, K, plan_bits, fit < 1 ? 1 : fit > (size_t)kMaxSplits ? kMaxSplits : (int)fit);
         }
         // (the partial sums of a tile are addressed with 32-bit byte offsets that must stay below 2^31)
         if (plan.splits > 1 && N * 512 > (int64_t)INT32_MAX) plan = plan_from_variant(M, N, K, plan_bits & 0xff00, 1);
@@ -2723,11 +2764,14 @@ int mi355x_fp8_rowwise_gemm_noalloc(const void* a, const void* b, const float* a
     return fail(MI355X_FP8_EINVAL, "unknown variant 0x%x", variant);
   // host arithmetic only up to here: an oversized request is turned away before any device call
   const size_t need = mi355x_fp8_rowwise_workspace_bytes(M, N, K, variant);
-  if (need > kScratchBytes)
+  // A plan the buffer cannot hold is refused only when the caller named its split factor; left to
+  // the library, the call runs the cheapest plan whose partial sums fit the buffer, as the workspace
+  // form does with a workspace that is too small.
+  if (need > kScratchBytes && ((variant >> 16) & 0xff))
     return fail(MI355X_FP8_ENOTSUP,
-                "the plan for %lldx%lldx%lld needs %zu bytes of split-K scratch, the built-in buffer holds %zu; "
+                "split-K factor %d on %lldx%lldx%lld needs %zu bytes of scratch, the built-in buffer holds %zu; "
                 "call mi355x_fp8_rowwise_gemm with a workspace of that size instead",
-                (long long)M, (long long)N, (long long)K, need, kScratchBytes);
+                (variant >> 16) & 0xff, (long long)M, (long long)N, (long long)K, need, kScratchBytes);
   void* ws = nullptr;
   if (need) {
     if (const int ss = scratch_of_current_device(&ws)) return ss;

@@ -16,6 +16,7 @@ def _require_gpu(t: torch.Tensor, name: str) -> None:
             f"{name} is on {t.device}: the MI355X backend only runs on a ROCm device "
             "(there is no CPU fallback)"
         )
+    _lib.init_device(t.device.index if t.device.index is not None else torch.cuda.current_device())
 
 
 def _stream_ptr() -> int:
