@@ -39,6 +39,16 @@ TRAFFIC_FILES = {  # written by `python -m tritonbench_amd.harness.traffic` from
 }
 LLAMA3_70B_NK = [(10240, 8192), (8192, 8192), (57344, 8192), (8192, 28672)]
 LLAMA3_70B_M = [1, 32, 128, 1024, 4096]
+# the reference operator's own default sweep (tritonbench/operators/fp8_gemm_rowwise/operator.py:107-128);
+# entry 7, (16, 13312, 13312), is the shape of its one stored run configuration
+# (benchmarks/run_config/fp8_gemm_rowwise_fwd.yaml:1-3)
+REFERENCE_BUILTIN_SHAPES = [
+    (1, 2304, 2048), (1, 8192, 16384), (4, 4096, 2304), (4, 13312, 2048), (8, 2304, 2304),
+    (8, 8192, 6656), (16, 4096, 6656), (16, 13312, 13312), (32, 2304, 16384), (32, 8192, 13312),
+    (64, 4096, 2048), (64, 13312, 2048), (128, 2304, 6656), (128, 8192, 2304), (2048, 8192, 2048),
+    (2048, 13312, 6656), (4096, 2304, 13312), (4096, 13312, 2304), (16384, 4096, 16384),
+    (16384, 8192, 13312),
+]
 
 
 def source_sha() -> str:
@@ -133,6 +143,42 @@ def time_steps(sets, workspace, steps, warmup):
     end.record(stream)
     torch.cuda.synchronize()
     return start.elapsed_time(end) / steps
+
+
+def time_steps_graph(sets, workspace, steps, warmup, preheat_ms, replays=5):
+    """The headline's timed region as the reference operator times its backends
+    (use_cuda_graphs, tritonbench/operators/fp8_gemm_rowwise/operator.py:156): exactly `steps` calls
+    recorded into one HIP graph; `warmup` eager calls first, then untimed replays for `preheat_ms`
+    (recording the graph leaves the device idle for tens of milliseconds and its clock falls back);
+    then ONE replay between two events on the graph's stream, synchronised on both sides. Returns
+    (ms per step of that replay, [ms per step of `replays` further replays])."""
+    side = torch.cuda.Stream()
+    with torch.cuda.stream(side):
+        for i in range(max(warmup, 1)):
+            launch(sets[i % len(sets)], workspace)
+        torch.cuda.synchronize()
+        g = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g, stream=side):
+            for i in range(steps):
+                launch(sets[i % len(sets)], workspace)
+        t0 = time.perf_counter()
+        g.replay()
+        while (time.perf_counter() - t0) * 1e3 < preheat_ms:
+            g.replay()
+        torch.cuda.synchronize()
+
+        def one():
+            start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            torch.cuda.synchronize()
+            start.record(side)
+            g.replay()
+            end.record(side)
+            torch.cuda.synchronize()
+            return start.elapsed_time(end) / steps
+
+        timed = one()
+        more = [one() for _ in range(replays)]
+    return timed, more
 
 
 def time_graph(call, steps, min_replay_ms=6.0, preheat_ms=30.0, replays=5):
@@ -307,36 +353,62 @@ def time_blockwise(m, n, k, dev, steps=30):
                 frac=flops / ms / 1e9 / PEAK_FP8_TFLOPS)
 
 
-def cpu_baseline(s, what, budget_s=12.0, max_calls=5):
-    """The oracle (fp32 dequantise + torch.matmul) on host cores, on the same operands."""
+def cpu_weight(s):
+    """The weight of operand set `s` on the host, dequantised to fp32 (the first half of the CPU path);
+    returns (tensor, seconds). Rows of one (N, K) pair share it across their M sweep."""
+    from oracle import fp8_rowwise as orc
+
+    _, wq, _, ws, _, _ = s
+    hwq, hws = wq.cpu(), ws.cpu()
+    orc.dequantize(hwq[:64], hws[:64])  # (pages the conversion code in)
+    t0 = time.perf_counter()
+    w = orc.dequantize(hwq, hws)
+    return w, time.perf_counter() - t0
+
+
+def cpu_baseline(s, what, budget_s=12.0, max_calls=5, weight=None):
+    """The oracle (fp32 dequantise + torch.matmul) on host cores, on the same operands, the two
+    halves timed separately. `weight` = (dequantised fp32 weight, seconds it took) from cpu_weight()
+    when several rows share one weight: its time is charged to every row as if it had been redone."""
     from oracle import fp8_rowwise as orc
 
     xq, wq, xs, ws, b, _ = s
-    hxq, hwq, hxs, hws = xq.cpu(), wq.cpu(), xs.cpu(), ws.cpu()
+    hxq, hxs = xq.cpu(), xs.cpu()
     hb = None if b is None else b.cpu()
     m, k = hxq.shape
-    n = hwq.shape[0]
+    n = wq.shape[0]
+    flops = 2 * m * n * k + (2 * m * n if b is not None else 0)
+    if weight is None:
+        weight = cpu_weight(s)
+    w, w_seconds = weight
     t0 = time.perf_counter()
-    orc.dequant_matmul(hxq, hwq, hxs, hws, hb)  # warm-up (also pages in the BLAS)
+    a = orc.dequantize(hxq, hxs)
+    deq = w_seconds + (time.perf_counter() - t0)
+    # (a call that takes a second is timed once; short ones take the best of a few after a warm-up)
+    t0 = time.perf_counter()
+    orc.dequant_matmul_rows(a, w, hb)
     first = time.perf_counter() - t0
-    times, spent = [], 0.0
-    while spent < budget_s and len(times) < max_calls:
+    times, spent = [first] if first > 0.5 else [], first
+    while spent < budget_s and len(times) < max_calls and first <= 0.5 * budget_s:
         t0 = time.perf_counter()
-        orc.dequant_matmul(hxq, hwq, hxs, hws, hb)
+        orc.dequant_matmul_rows(a, w, hb)
         dt = time.perf_counter() - t0
         times.append(dt)
         spent += dt
-    best = min(times) if times else first
-    flops = 2 * m * n * k + (2 * m * n if b is not None else 0)
+    mm = min(times) if times else first
+    total = deq + mm
     return {
-        "value": flops / best / 1e12,
+        "value": flops / total / 1e12,
         "unit": "TFLOP/s",
-        "gbps": (m * k + n * k + 2 * m * n) / best / 1e9,
-        "ms": best * 1e3,
+        "gbps": (m * k + n * k + 2 * m * n) / total / 1e9,
+        "ms": total * 1e3,
+        "dequant_ms": deq * 1e3,
+        "matmul_ms": mm * 1e3,
         "cores": torch.get_num_threads(),
+        "cpu_count": os.cpu_count(),
         "kind": "port",
-        "sample": f"full {what} workload, best of {len(times)} calls after 1 warm-up ({best:.4f} s/call, "
-                  f"dequantise included, host cpu_count {os.cpu_count()})",
+        "sample": f"full {what} workload: fp32 dequantise of both operands ({deq:.4f} s) + torch.matmul, bias and bf16 rounding "
+                  f"({mm:.4f} s, best of {max(len(times), 1)} call(s))",
     }
 
 
@@ -420,8 +492,19 @@ def main():
     head_sets, head_ws = make_sets(m, make_weights(n, k, 1.0, False, dev, 1), 1.0, dev)
     torch.cuda.synchronize()
     preheat(head_sets, head_ws, args.preheat_ms)
-    ms = time_steps(head_sets, head_ws, args.steps, args.warmup)
+    ms, replays_ms = time_steps_graph(head_sets, head_ws, args.steps, args.warmup, args.preheat_ms)
     head = figures(m, n, k, False, ms)
+    # the same steps as plain launches on a stream (what a caller without a graph sees: the gap between
+    # two dependent launches is several microseconds longer than between two nodes of a graph)
+    ms_stream = time_steps(head_sets, head_ws, args.steps, args.warmup)
+    # one launch with clock readings, while the device is still under load: cycles belong to the kernel,
+    # the clock to the box (and to each XCD: the slowest one ends the launch)
+    try:
+        from tritonbench_amd import ops
+
+        clocks = ops.fp8_gemm_rowwise_clocks(*head_sets[0][:4], head_sets[0][5], workspace=head_ws)
+    except Exception as e:  # noqa: BLE001 - a diagnostic: its failure must not cost the line
+        clocks = {"error": f"{type(e).__name__}: {e}"}
     traffic, traffic_note = measured_traffic("tiled")
 
     line = {
@@ -433,12 +516,18 @@ def main():
         "warmup": args.warmup,
         "preheat_ms": args.preheat_ms,
         "ms_per_step": ms,
+        "us_min": min(replays_ms + [ms]) * 1e3,
+        "us_median": statistics.median(replays_ms + [ms]) * 1e3,
+        "ms_per_step_stream_launches": ms_stream,
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
         "dtype": "fp8_e4m3fn x fp8_e4m3fn -> f32 accumulate -> bf16",
         "data": "synthetic (seeded N(0,1) fp32, row-wise e4m3fn quantised on device)",
-        "config": {"workload": "c2_square M=N=K=8192, row-wise scales, no bias, bf16 out", "variant": "tiled"},
+        "config": {"workload": "c2_square M=N=K=8192, row-wise scales, no bias, bf16 out", "variant": "tiled",
+                   "launch": "the timed steps are one replay of a HIP graph holding exactly `steps` calls, as the reference "
+                             "operator times its backends (use_cuda_graphs); ms_per_step_stream_launches is the same "
+                             "count of plain launches"},
         "roofline": {
             "bound": "mfma",
             "achieved": head["tflops"],
@@ -450,6 +539,11 @@ def main():
             "traffic": traffic,
             **traffic_note,
         },
+        # What part of the fraction is the kernel's and what the box's: the MFMA instructions of one launch
+        # occupy every SIMD for mfma_cycles; a workgroup takes cycles_per_workgroup_* shader cycles for
+        # them; the XCDs run at clocks of their own (the peak is quoted at 2.4 GHz) and the slowest ends
+        # the launch.
+        "clock": {**(clocks or {}), "mfma_cycles": 2 * m * n * k // (2048 * 1024), "peak_quoted_at_ghz": 2.4},
     }
 
     if not args.no_extra:
@@ -505,6 +599,13 @@ def main():
             attempt(f"c5_ragged_bias_{rm}x{rn}x{rk}", lambda: c5(rm, rn, rk))
         attempt("c2_square_8192_graph", lambda: gemm_row(m, head_sets, head_ws, 20))
 
+        def c2_cold():
+            # five operand sets (1.9 GB: A, B and C of each are out of every cache when their turn comes again)
+            cs, cws = make_sets(m, make_weights(n, k, 1.0, False, dev, 5), 1.0, dev)
+            return gemm_row(m, cs, cws, 20)
+
+        attempt("c2_square_8192_cold", c2_cold)
+
         def c1():
             # C1: the reference's CPU-runnable plumbing case, here on the device with the host figure beside it
             ps, pws = make_sets(128, make_weights(256, 512, 1.0, False, dev, 1), 1.0, dev)
@@ -515,22 +616,36 @@ def main():
 
         attempt("c1_plumbing_128x256x512", c1)
 
-        def c4(lm, ln, lk, weights):
+        def c4(lm, ln, lk, weights, host_weight):
             ls, lws = make_sets(lm, weights, 0.02, dev)
-            return gemm_row(lm, ls, lws, 30 if lm < 1024 else 10)
+            row = gemm_row(lm, ls, lws, 30 if lm < 1024 else 10)
+            if host_weight is not None:
+                row["cpu_baseline"] = cpu_baseline(ls[0], f"{lm}x{ln}x{lk}", budget_s=1.0, max_calls=3, weight=host_weight)
+            return row
 
-        # C4: Llama-3-70B projections, sigma 0.02; the weight copies of an (N, K) pair serve its whole M sweep
+        # C4: Llama-3-70B projections, sigma 0.02; the weight copies of an (N, K) pair serve its whole M sweep,
+        # and so does the fp32 copy of the first one on the host for the CPU figure beside every row
         for (ln, lk) in LLAMA3_70B_NK:
             try:
                 weights = make_weights(ln, lk, 0.02, False, dev, copies_for(ln, lk))
+                host_weight = cpu_weight((None, weights[0][0], None, weights[0][1], None, None)) if cpu else None
             except Exception as e:  # noqa: BLE001 - the weights did not fit or could not be made: every row of the pair says so
                 for lm in LLAMA3_70B_M:
                     configs[f"c4_llama70b_{lm}x{ln}x{lk}"] = {"error": f"{type(e).__name__}: {e}"}
                 print(f"bench.py: weights {ln}x{lk} failed: {type(e).__name__}: {e}", file=sys.stderr, flush=True)
                 continue
             for lm in LLAMA3_70B_M:
-                attempt(f"c4_llama70b_{lm}x{ln}x{lk}", lambda: c4(lm, ln, lk, weights))
-            del weights
+                attempt(f"c4_llama70b_{lm}x{ln}x{lk}", lambda: c4(lm, ln, lk, weights, host_weight))
+            del weights, host_weight
+            torch.cuda.empty_cache()
+
+        # the reference operator's own default sweep (no CPU figure: these are not configurations of the baseline)
+        def builtin(bm, bn, bk):
+            bs, bws = make_sets(bm, make_weights(bn, bk, 1.0, False, dev, copies_for(bn, bk)), 1.0, dev)
+            return gemm_row(bm, bs, bws, 30 if bm < 1024 else 10)
+
+        for (bm, bn, bk) in REFERENCE_BUILTIN_SHAPES:
+            attempt(f"ref_builtin_{bm}x{bn}x{bk}", lambda: builtin(bm, bn, bk))
             torch.cuda.empty_cache()
         attempt("grouped_g4_8192x4096x4096", lambda: time_grouped(4, 8192, 4096, 4096, dev))
         attempt("grouped_g16_8192x8192x8192", lambda: time_grouped(16, 8192, 8192, 8192, dev, steps=20))
@@ -548,6 +663,7 @@ def main():
 
     if not args.no_cpu_baseline:
         line["cpu_baseline"] = cpu_baseline(head_sets[0], "M=N=K=8192")
+        line["vs_cpu_baseline"] = line["value"] / line["cpu_baseline"]["value"]
 
     print(json.dumps(line))
 

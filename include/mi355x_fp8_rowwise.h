@@ -153,6 +153,27 @@ int mi355x_fp8_rowwise_gemm_ex(const void* a, const void* b,
                                int variant, void* stream);
 
 /*
+ * mi355x_fp8_rowwise_gemm with clock readings, for benchmarks that want to tell a kernel's cycles
+ * from the clock it ran at (the sustained clock under matrix load differs from box to box and
+ * moves with power). It has no counterpart in the reference. Same operands and results as
+ * mi355x_fp8_rowwise_gemm; in addition every workgroup g of a TILED-family launch writes four
+ * 64-bit readings to stamps[4*g .. 4*g+3]: the shader clock counter at its first and after its
+ * last instruction, and the constant 100 MHz counter at the same two points. Workgroups that had
+ * no work, and launches of the other kernel families, write nothing: clear the buffer first and
+ * skip groups whose first reading is zero. max(end) - min(start) over the groups is the launch in
+ * shader cycles, the same difference of the 100 MHz readings its duration.
+ * `stamps` is device memory of at least MI355X_FP8_STAMP_ENTRIES 64-bit entries, 8-byte aligned.
+ */
+#define MI355X_FP8_STAMP_ENTRIES 2048
+int mi355x_fp8_rowwise_gemm_stamped(const void* a, const void* b,
+                                    const float* a_scale, const float* b_scale,
+                                    const void* bias, void* c,
+                                    int64_t M, int64_t N, int64_t K,
+                                    int64_t lda, int64_t ldb, int64_t ldc,
+                                    void* workspace, size_t workspace_bytes,
+                                    int variant, uint64_t* stamps, size_t stamp_entries, void* stream);
+
+/*
  * mi355x_fp8_rowwise_gemm for callers that can neither allocate nor bring a workspace: code
  * under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc. It has no
  * counterpart in the reference (there every backend allocates through PyTorch). Same operands,

@@ -111,6 +111,33 @@ def test_c4_llama70b_projections(gpu_device, name):
         del out, dxq, dxs
 
 
+def _builtin_shapes():
+    from tritonbench_amd.operators.fp8_gemm_rowwise.operator import BUILDIN_SHAPES
+
+    return list(BUILDIN_SHAPES)
+
+
+@pytest.mark.parametrize("m,n,k", _builtin_shapes())
+def test_reference_builtin_shapes(gpu_device, m, n, k):
+    """The reference operator's own default sweep (tritonbench/operators/fp8_gemm_rowwise/operator.py:107-128;
+    (16, 13312, 13312) is the shape of its stored run configuration): every row for M <= 128, a sample
+    of rows above, against the oracle."""
+    print(f"builtin m={m} n={n} k={k} variant={ops.select_variant(m, n, k)}", flush=True)
+    xq, wq, xs, ws, _ = orc.make_inputs(m, n, k, 1.0, False)
+    dxq, dwq, dxs, dws = _gpu(gpu_device, xq, wq, xs, ws)
+    out = ops.fp8_gemm_rowwise(dxq, dwq, dxs, dws)
+    torch.cuda.synchronize()
+    rows = torch.arange(m) if m <= 128 else _sample_rows(m, 32)
+    _check_rows(out, xq, wq, xs, ws, None, rows, 1.0)
+    if m <= 128:
+        # the other kernel family on the same operands
+        other = _lib.VARIANT_TILED if ops.select_variant(m, n, k) == _lib.VARIANT_SKINNY else _lib.VARIANT_SKINNY
+        if other == _lib.VARIANT_TILED or _lib.skinny_family_takes(m, n):
+            out2 = ops.fp8_gemm_rowwise(dxq, dwq, dxs, dws, variant=other)
+            torch.cuda.synchronize()
+            torch.testing.assert_close(out2, out, rtol=RTOL, atol=ATOL)
+
+
 def test_output_beyond_2_to_31_elements(gpu_device):
     # 32800 x 65600 bf16 = 2.15e9 elements (4.3 GB): row offsets into C pass both 2^31 elements
     # and 2^32 bytes; K is one step, so the case costs a few hundred microseconds of GPU time

@@ -27,7 +27,12 @@ SHAPES = [(32, 8192, 8192, False), (64, 8192, 8192, False), (128, 8192, 8192, Fa
           (1, 8192, 8192, False), (1, 10240, 8192, False), (1, 57344, 8192, False), (1, 8192, 28672, False),
           (32, 57344, 8192, False), (32, 8192, 28672, False), (128, 57344, 8192, False),
           # one tile row of 256x256 tiles with streamed B; several tile rows of the smaller configurations
-          (256, 57344, 8192, False), (512, 16384, 16384, False)]
+          (256, 57344, 8192, False), (512, 16384, 16384, False),
+          # decode-sized rows of the reference operator's own default sweep (operator.py:107-128); the
+          # first is the shape of its stored run configuration
+          (16, 13312, 13312, False), (1, 8192, 16384, False), (4, 13312, 2048, False), (8, 8192, 6656, False),
+          (16, 4096, 6656, False), (32, 2304, 16384, False), (32, 8192, 13312, False), (64, 13312, 2048, False),
+          (128, 2304, 6656, False), (128, 8192, 2304, False)]
 
 
 def _time_us(dev, m, n, k, bias, variant, sets):

@@ -35,6 +35,7 @@ def skinny_family_takes(m: int, n: int) -> bool:
 
 NUM_TILE_CONFIGS = 6
 NOALLOC_SCRATCH_BYTES = 64 << 20
+STAMP_ENTRIES = 2048
 NUM_GROUPED_TILE_CONFIGS = 3
 
 
@@ -71,6 +72,12 @@ SIGNATURES = {
         [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int,
          c_int64, c_int64, c_int64, c_int64, c_int64, c_int64,
          c_void_p, c_size_t, c_int, c_void_p],
+    ),
+    "mi355x_fp8_rowwise_gemm_stamped": (
+        c_int,
+        [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
+         c_int64, c_int64, c_int64, c_int64, c_int64, c_int64,
+         c_void_p, c_size_t, c_int, c_void_p, c_size_t, c_void_p],
     ),
     "mi355x_fp8_rowwise_gemm_noalloc": (
         c_int,

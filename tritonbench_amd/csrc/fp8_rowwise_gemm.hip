@@ -72,6 +72,12 @@ struct GemmParams {
   const int32_t* m_sizes;
   int groups;
   int out_f16;  // C holds IEEE binary16 instead of bf16 (same size, same stores)
+  // tiled kernel, plain form: reciprocals of the two run-time divisors of the tile walk (the number
+  // of tiles, and the tiles of a full group of tile rows), prepared on the host: see fast_div()
+  uint32_t div_tiles_mul, div_tiles_shift, div_group_mul, div_group_shift;
+  // tiled kernel: where every workgroup leaves its start and end readings of the shader clock and of
+  // the constant 100 MHz clock (4 values per workgroup), or nullptr
+  unsigned long long* stamps;
 };
 
 // Where a tile sits: rows [m0, m_end) of A and C it may touch, first column, group.
@@ -140,15 +146,34 @@ __device__ __forceinline__ TileWalk make_walk(int total_tiles) {
   return w;
 }
 
-__device__ __forceinline__ void tile_coords(int t, int tiles_m, int tiles_n, int group_m,
+// Division of a wave-uniform n < 2^31 by a run-time divisor d whose reciprocal the host prepared:
+// mul = ceil(2^shift / d), shift = 31 + ceil(log2 d), and then floor(n / d) = (n * mul) >> shift
+// exactly (mul * d lies within 2^(shift-31) of 2^shift). Three scalar instructions where the
+// compiler's expansion of a division is a few dozen, on the path that moves a load cursor from one
+// tile to the next in the middle of the K pipeline.
+__device__ __forceinline__ int fast_div(int n, uint32_t mul, uint32_t shift) {
+  return (int)(uint32_t)(((uint64_t)(uint32_t)n * mul) >> shift);
+}
+inline void make_fast_div(uint32_t d, uint32_t& mul, uint32_t& shift) {
+  int l = 0;
+  while ((1ull << l) < d) ++l;
+  shift = 31u + (uint32_t)l;
+  mul = (uint32_t)(((1ull << shift) + d - 1) / d);
+}
+
+constexpr int kGroupM = 4;  // tile rows walked together (a group); the last group may hold fewer
+
+// tile number -> tile row and column in grouped order (kGroupM tile rows at a time, column-major inside a group)
+__device__ __forceinline__ void tile_coords(int t, int tiles_m, int tiles_n, uint32_t group_mul, uint32_t group_shift,
                                             int& tm, int& tn) {
-  const int per_group = group_m * tiles_n;
-  const int g = t / per_group;
-  const int first_m = g * group_m;
-  const int gsz = min(tiles_m - first_m, group_m);
+  const int per_group = kGroupM * tiles_n;
+  const int g = fast_div(t, group_mul, group_shift);
+  const int first_m = g * kGroupM;
+  const int gsz = min(tiles_m - first_m, kGroupM);
   const int in_g = t - g * per_group;
-  tm = first_m + in_g % gsz;
-  tn = in_g / gsz;
+  // in_g / gsz for gsz in 1..4
+  tn = gsz == 4 ? in_g >> 2 : gsz == 3 ? fast_div(in_g, 0xAAAAAAABu, 33) : gsz == 2 ? in_g >> 1 : in_g;
+  tm = first_m + in_g - tn * gsz;
 }
 
 // ------------------------------------------------------------------------------------
@@ -308,6 +333,13 @@ void gemm_tiled_kernel(GemmParams p) {
 
   extern __shared__ __attribute__((aligned(1024))) uint8_t lds[];
 
+  // (diagnostic launches only: the shader clock and the constant 100 MHz clock at this workgroup's start)
+  unsigned long long stamp_cycles = 0, stamp_ticks = 0;
+  if (p.stamps) {
+    stamp_cycles = __builtin_readcyclecounter();
+    stamp_ticks = __builtin_amdgcn_s_memrealtime();
+  }
+
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int wm = wave / WAVES_N, wn = wave % WAVES_N;
@@ -350,8 +382,16 @@ void gemm_tiled_kernel(GemmParams p) {
   const int k_full = p.K / kStepK;             // whole 128-byte steps
   const int k_tail = p.K - k_full * kStepK;    // 0 or a multiple of 16
   const int k_steps = k_full + (k_tail ? 1 : 0);
-  auto item_split = [&](int li) { return (walk.chunk_begin + li) / total_tiles; };
-  auto item_tile = [&](int li) { return (walk.chunk_begin + li) % total_tiles; };
+  // (the grouped form counts its tiles on the device and divides the ordinary way; an unsplit launch has
+  // nothing to divide)
+  auto item_split = [&](int li) {
+    const int t = walk.chunk_begin + li;
+    return GROUPED ? t / total_tiles : p.splits == 1 ? 0 : fast_div(t, p.div_tiles_mul, p.div_tiles_shift);
+  };
+  auto item_tile = [&](int li) {
+    const int t = walk.chunk_begin + li;
+    return GROUPED ? t % total_tiles : p.splits == 1 ? t : t - fast_div(t, p.div_tiles_mul, p.div_tiles_shift) * total_tiles;
+  };
   auto split_begin = [&](int sp) { return sp * p.steps_per_split; };
   auto split_end = [&](int sp) { return min((sp + 1) * p.steps_per_split, k_steps); };
   int total_steps = 0;
@@ -364,7 +404,7 @@ void gemm_tiled_kernel(GemmParams p) {
     const int tile = item_tile(li);
     if (!GROUPED) {
       int tm, tn;
-      tile_coords(tile, p.tiles_m, p.tiles_n, p.group_m, tm, tn);
+      tile_coords(tile, p.tiles_m, p.tiles_n, p.div_group_mul, p.div_group_shift, tm, tn);
       return TileLoc{tm * BM, p.M, tn * BN, 0};
     }
     while (tile >= w.tile_end && w.group + 1 < p.groups) {
@@ -1021,6 +1061,13 @@ void gemm_tiled_kernel(GemmParams p) {
     read_first_half();  // of the next item's first step (landed before this item's last barrier)
   }
   __builtin_amdgcn_s_waitcnt(0x0070);  // the trailing dummy loads must land before LDS is released
+  if (p.stamps && threadIdx.x == 0) {
+    unsigned long long* out = p.stamps + 4 * (size_t)blockIdx.x;
+    out[0] = stamp_cycles;
+    out[1] = __builtin_readcyclecounter();
+    out[2] = stamp_ticks;
+    out[3] = __builtin_amdgcn_s_memrealtime();
+  }
 }
 
 // Second pass of a split-K launch: sums the splits' partials in a fixed order (results do not
@@ -2435,8 +2482,11 @@ int launch_tiled(GemmParams p, hipStream_t stream) {
   // grouped: the group sizes live on the device; every group adds at most one partial tile row
   p.tiles_m = GROUPED ? p.M / BM + p.groups : (p.M + BM - 1) / BM;
   p.tiles_n = (p.N + BN - 1) / BN;
-  p.group_m = 4;
+  p.group_m = kGroupM;
+  make_fast_div((uint32_t)p.tiles_m * (uint32_t)p.tiles_n, p.div_tiles_mul, p.div_tiles_shift);
+  make_fast_div((uint32_t)kGroupM * (uint32_t)p.tiles_n, p.div_group_mul, p.div_group_shift);
   const long total = (long)p.tiles_m * p.tiles_n * p.splits;
+  if (total > (long)INT32_MAX) return fail(MI355X_FP8_ENOTSUP, "more than 2^31-1 work items");
   const long slots = (long)kNumCu * tiled_wgs_per_cu(BM, BN, BLOCKSCALE, DIST);
   long grid = total < slots ? ((total + kNumXcd - 1) / kNumXcd) * kNumXcd : slots;
   constexpr auto kern = gemm_tiled_kernel<BM, BN, WAVES_M, WAVES_N, KTAIL, EPI, GROUPED, BLOCKSCALE, DIST, STREAM_B>;
@@ -2599,6 +2649,10 @@ int launch_narrow_for(const GemmParams& p, hipStream_t s) {
   return f.nb == 1 ? launch_narrow<2, 1>(p, s) : launch_narrow<2, 2>(p, s);
 }
 
+int run_gemm(const void* a, const void* b, const float* a_scale, const float* b_scale, const void* bias, void* c,
+             int out_type, int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldb, int64_t ldc, void* workspace,
+             size_t workspace_bytes, int variant, void* stream, unsigned long long* stamps);
+
 }  // namespace
 
 extern "C" {
@@ -2644,6 +2698,27 @@ int mi355x_fp8_rowwise_gemm_ex(const void* a, const void* b, const float* a_scal
                                const void* bias, void* c, int out_type, int64_t M, int64_t N, int64_t K,
                                int64_t lda, int64_t ldb, int64_t ldc, void* workspace, size_t workspace_bytes,
                                int variant, void* stream) {
+  return run_gemm(a, b, a_scale, b_scale, bias, c, out_type, M, N, K, lda, ldb, ldc, workspace, workspace_bytes, variant,
+                  stream, nullptr);
+}
+
+int mi355x_fp8_rowwise_gemm_stamped(const void* a, const void* b, const float* a_scale, const float* b_scale,
+                                    const void* bias, void* c, int64_t M, int64_t N, int64_t K, int64_t lda,
+                                    int64_t ldb, int64_t ldc, void* workspace, size_t workspace_bytes, int variant,
+                                    uint64_t* stamps, size_t stamp_entries, void* stream) {
+  if (!stamps || stamp_entries < (size_t)MI355X_FP8_STAMP_ENTRIES)
+    return fail(MI355X_FP8_EINVAL, "stamps must hold %d entries (got %zu)", MI355X_FP8_STAMP_ENTRIES, stamps ? stamp_entries : (size_t)0);
+  if (reinterpret_cast<uintptr_t>(stamps) & 7) return fail(MI355X_FP8_EINVAL, "misaligned stamps pointer");
+  return run_gemm(a, b, a_scale, b_scale, bias, c, MI355X_FP8_OUT_BF16, M, N, K, lda, ldb, ldc, workspace, workspace_bytes,
+                  variant, stream, reinterpret_cast<unsigned long long*>(stamps));
+}
+
+}  // extern "C"
+
+namespace {
+int run_gemm(const void* a, const void* b, const float* a_scale, const float* b_scale, const void* bias, void* c,
+             int out_type, int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldb, int64_t ldc, void* workspace,
+             size_t workspace_bytes, int variant, void* stream, unsigned long long* stamps) {
   if (out_type != MI355X_FP8_OUT_BF16 && out_type != MI355X_FP8_OUT_F16)
     return fail(MI355X_FP8_EINVAL, "unknown output type %d", out_type);
   int st = check_shape(M, N, K);
@@ -2688,6 +2763,7 @@ int mi355x_fp8_rowwise_gemm_ex(const void* a, const void* b, const float* a_scal
   p.tiles_m = p.tiles_n = 0; p.group_m = 1;
   p.splits = 1; p.steps_per_split = k_steps_of(K); p.partial = nullptr;
   p.m_sizes = nullptr; p.groups = 0; p.out_f16 = out_type == MI355X_FP8_OUT_F16;
+  p.div_tiles_mul = p.div_tiles_shift = p.div_group_mul = p.div_group_shift = 0; p.stamps = stamps;
   hipStream_t s = (hipStream_t)stream;
 
   switch (variant) {
@@ -2754,6 +2830,9 @@ int mi355x_fp8_rowwise_gemm_ex(const void* a, const void* b, const float* a_scal
       return fail(MI355X_FP8_EINVAL, "unknown variant %d", variant);
   }
 }
+}  // namespace
+
+extern "C" {
 
 int mi355x_fp8_rowwise_gemm_noalloc(const void* a, const void* b, const float* a_scale, const float* b_scale,
                                     const void* bias, void* c, int64_t M, int64_t N, int64_t K, int64_t lda,
@@ -2813,6 +2892,7 @@ int mi355x_fp8_rowwise_grouped_gemm(const void* a, const void* b, const float* a
   p.tiles_m = p.tiles_n = 0; p.group_m = 1;
   p.splits = 1; p.steps_per_split = k_steps_of(K); p.partial = nullptr;
   p.m_sizes = m_sizes; p.groups = (int)G; p.out_f16 = 0;
+  p.div_tiles_mul = p.div_tiles_shift = p.div_group_mul = p.div_group_shift = 0; p.stamps = nullptr;
   hipStream_t s = (hipStream_t)stream;
   // Large tiles when an average group fills most of one and there are enough of them for every
   // CU, small tiles otherwise (the group sizes themselves are on the device; M / G is what the
@@ -2856,6 +2936,7 @@ int mi355x_fp8_blockwise_gemm(const void* a, const void* b, const float* a_scale
   p.tiles_m = p.tiles_n = 0; p.group_m = 1;
   p.splits = 1; p.steps_per_split = k_steps_of(K); p.partial = nullptr;
   p.m_sizes = nullptr; p.groups = 0; p.out_f16 = 0;
+  p.div_tiles_mul = p.div_tiles_shift = p.div_group_mul = p.div_group_shift = 0; p.stamps = nullptr;
   hipStream_t s = (hipStream_t)stream;
   // 128x128 tiles: with 256x128 tiles (64 more accumulators and 64 more partial products per
   // lane) the fold no longer fits the 256 registers VALU instructions can address

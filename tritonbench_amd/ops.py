@@ -107,6 +107,47 @@ def fp8_gemm_rowwise(
     return out
 
 
+def fp8_gemm_rowwise_clocks(xq, wq, x_scale, w_scale, out, workspace=None, variant: int = _lib.VARIANT_AUTO) -> Optional[dict]:
+    """One launch of fp8_gemm_rowwise through mi355x_fp8_rowwise_gemm_stamped, read back: what the
+    launch took in shader cycles and at which clock every XCD ran it (workgroup g runs on XCD g % 8;
+    each XCD has a clock of its own). Returns None when the plan is not of the tiled family (only
+    that one records readings). Synchronises; for benchmarks, outside their timed regions."""
+    lib = _lib.load()
+    for t, name in ((xq, "xq"), (wq, "wq"), (x_scale, "x_scale"), (w_scale, "w_scale"), (out, "out")):
+        _require_gpu(t, name)
+    m, k = xq.shape
+    n = wq.shape[0]
+    stamps = torch.zeros(_lib.STAMP_ENTRIES, dtype=torch.int64, device=xq.device)
+    ws_bytes = workspace.numel() * workspace.element_size() if workspace is not None else 0
+    st = lib.mi355x_fp8_rowwise_gemm_stamped(
+        xq.data_ptr(), wq.data_ptr(), x_scale.data_ptr(), w_scale.data_ptr(), None, out.data_ptr(),
+        m, n, k, xq.stride(0), wq.stride(0), out.stride(0),
+        workspace.data_ptr() if workspace is not None else None, ws_bytes, variant,
+        stamps.data_ptr(), _lib.STAMP_ENTRIES, _stream_ptr(),
+    )
+    _lib.check(st, "mi355x_fp8_rowwise_gemm_stamped")
+    torch.cuda.synchronize()
+    t = stamps.cpu().view(-1, 4)
+    t = t[t[:, 0] != 0]
+    if t.numel() == 0:
+        return None
+    groups = torch.nonzero(stamps.cpu().view(-1, 4)[:, 0] != 0).flatten()
+    cycles = (t[:, 1] - t[:, 0]).double()
+    ticks = (t[:, 3] - t[:, 2]).double()          # 100 MHz
+    ghz = cycles / (ticks * 10.0)
+    per_xcd = [float(ghz[(groups % 8) == x].mean()) for x in range(8) if bool(((groups % 8) == x).any())]
+    return {
+        "workgroups": int(t.shape[0]),
+        "cycles_per_workgroup_mean": float(cycles.mean()),
+        "cycles_per_workgroup_max": float(cycles.max()),
+        "span_us": float((t[:, 3].max() - t[:, 2].min()).item()) / 100.0,
+        "xcd_clock_ghz": [round(v, 4) for v in per_xcd],
+        "clock_ghz_mean": float(ghz.mean()),
+        "clock_ghz_min_xcd": min(per_xcd),
+        "clock_ghz_max_xcd": max(per_xcd),
+    }
+
+
 def fp8_gemm_tensorwise(
     a: torch.Tensor,
     b: torch.Tensor,
