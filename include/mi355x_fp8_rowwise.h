@@ -67,9 +67,12 @@ extern "C" {
  * number of 128-byte K steps is reduced to it.
  */
 /* Skinny family only: bit 8 pins the form with one 16-row tile of B per workgroup (the general
- * one; M <= 64). Without it M <= 16 with N a multiple of 16 and K one of 2048, 4096, 6144, 8192 runs
- * the persistent form (one workgroup per CU walks a run of tiles with its share of A resident
- * in registers); every other shape runs the general form anyway. */
+ * one; M <= 64). Without a pin, M <= 16 with N a multiple of 16 runs a form that keeps A on chip for
+ * the whole launch (one 16-wave workgroup per CU): the pair form for N <= 8192 and any K <= 8192
+ * (at most two tiles of B per CU, A parked in LDS, a tile's loads issued in one burst), the
+ * persistent form for larger N with K one of 2048, 4096, 6144, 8192 (a run of tiles per CU, A in
+ * registers, rolling prefetch; also M <= 32 at K = 4096) - unless the narrow-tile form below is
+ * expected to be faster; every other shape runs the general form anyway. */
 #define MI355X_FP8_SKINNY_ONE_TILE      (1 << 8)
 /* Skinny family only: bit 9 pins the narrow-tile form (one workgroup per 32 or 64 columns of C owns
  * all of K). It takes M <= 64 and, in row blocks of 64 with 64-column tiles, 64 < M <= 256 when
@@ -77,6 +80,9 @@ extern "C" {
  * supported" otherwise. Without a pin the family runs whichever of its forms is expected to be
  * fastest. */
 #define MI355X_FP8_SKINNY_NARROW        (2 << 8)
+/* Skinny family only: bit 10 pins the forms that keep A on chip (pair or persistent, whichever takes
+ * the shape; "not supported" when neither does). */
+#define MI355X_FP8_SKINNY_RESIDENT      (4 << 8)
 #define MI355X_FP8_TILED_CONFIG(cfg)    ((((cfg) + 1) & 0xff) << 8)
 #define MI355X_FP8_TILED_SPLITS(s)      (((s) & 0xff) << 16)
 #define MI355X_FP8_NUM_TILE_CONFIGS     6

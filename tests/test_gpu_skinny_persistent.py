@@ -1,7 +1,9 @@
-"""Parity of the persistent skinny kernel (N % 16 == 0; M <= 16 with K in {2048, 4096, 6144, 8192},
-M <= 32 with K = 4096: two 16-row blocks of A resident in registers)
-with the CPU oracle, and against the one-tile-per-workgroup kernel it replaces on those shapes.
-Both are reached through the C ABI with the skinny family pinned. Needs an MI355X."""
+"""Parity of the skinny kernels that keep A on chip (N % 16 == 0) with the CPU oracle, and against
+the one-tile-per-workgroup kernel they replace on their shapes: the pair kernel (M <= 16, N <= 8192,
+any K <= 8192: at most two tiles of B per CU, A parked in LDS) and the persistent kernel (M <= 16
+with larger N and K in {2048, 4096, 6144, 8192}; M <= 32 with K = 4096: two 16-row blocks of A
+resident in registers). All are reached through the C ABI with the skinny family and the form
+pinned. Needs an MI355X."""
 import numpy as np
 import pytest
 import torch
@@ -15,7 +17,7 @@ pytestmark = pytest.mark.gpu
 RTOL = 1e-2  # the tolerance the path is specified to: rtol 1e-2 / atol 1e-2 on the bf16 output
 ATOL = 1e-2
 
-PERSISTENT = _lib.VARIANT_SKINNY
+PERSISTENT = _lib.VARIANT_SKINNY | _lib.SKINNY_RESIDENT  # pair or persistent kernel, whichever takes the shape
 ONE_TILE = _lib.VARIANT_SKINNY | _lib.SKINNY_ONE_TILE
 
 
@@ -56,6 +58,8 @@ SHAPES = [
     (1, 16, 2048, False), (16, 16, 8192, True), (7, 48, 4096, True), (16, 4096, 2048, False),
     (9, 4112, 6144, True), (16, 8192, 4096, False), (3, 8208, 2048, True), (16, 10240, 2048, True),
     (13, 2064, 8192, False), (16, 12304, 2048, False),
+    # beyond the pair kernel's two tiles per CU: the persistent kernel with one block of A
+    (9, 8208, 6144, True), (16, 16400, 8192, False), (5, 12304, 4096, True), (16, 20480, 6144, False),
     # two blocks of A (M = 17..32, K = 4096): last block full / one row / ragged
     (17, 16, 4096, True), (32, 8192, 4096, False), (25, 4112, 4096, True), (32, 10240, 4096, False),
     (20, 2064, 4096, True), (31, 12304, 4096, False),
@@ -66,7 +70,7 @@ SHAPES = [
 def test_persistent_kernel_against_oracle(gpu_device, m, n, k, bias):
     print(f"case m={m} n={n} k={k} bias={bias}", flush=True)
     if m <= 16:
-        assert ops.select_variant(m, n, k) == _lib.VARIANT_SKINNY  # what the automatic choice runs too
+        assert ops.select_variant(m, n, k) == _lib.VARIANT_SKINNY  # the family the automatic choice runs too
     xq, wq, xs, ws, b = orc.make_inputs(m, n, k, 1.0, bias)
     want = orc.dequant_matmul(xq, wq, xs, ws, b)
     out = _run(gpu_device, xq, wq, xs, ws, b, PERSISTENT)
@@ -78,7 +82,56 @@ def test_persistent_kernel_against_oracle(gpu_device, m, n, k, bias):
     _check_tight(other, xq, wq, xs, ws, b)
 
 
-@pytest.mark.parametrize("m,k", [(16, 2048), (5, 8192), (32, 4096), (19, 4096)])
+# m, n, k, bias for the pair kernel: K that is no multiple of 2048, of 128 (a partial last step down to one
+# 16-byte chunk), shorter than one step per wave (waves without any step), one to four steps per
+# wave; one tile, fewer tiles than CUs, exactly one and two per CU, one more than one per CU
+PAIR_SHAPES = [
+    (1, 16, 16, False), (16, 16, 144, True), (3, 48, 272, True), (16, 4096, 2304, False), (4, 4096, 2304, True),
+    (8, 2304, 2304, False), (16, 4096, 6656, True), (8, 8192, 6656, False), (1, 2304, 2048, True),
+    (16, 4112, 4112, True), (11, 8192, 8176, False), (16, 8192, 8192, True), (7, 8176, 2064, False),
+    (16, 512, 1040, True), (2, 8192, 128, False), (16, 6400, 5136, True),
+]
+
+
+@pytest.mark.parametrize("m,n,k,bias", PAIR_SHAPES)
+def test_pair_kernel_against_oracle(gpu_device, m, n, k, bias):
+    print(f"case m={m} n={n} k={k} bias={bias}", flush=True)
+    xq, wq, xs, ws, b = orc.make_inputs(m, n, k, 1.0, bias)
+    want = orc.dequant_matmul(xq, wq, xs, ws, b)
+    out = _run(gpu_device, xq, wq, xs, ws, b, PERSISTENT)
+    torch.testing.assert_close(out, want, rtol=RTOL, atol=ATOL)
+    _check_tight(out, xq, wq, xs, ws, b)
+    other = _run(gpu_device, xq, wq, xs, ws, b, ONE_TILE)
+    torch.testing.assert_close(other, out, rtol=RTOL, atol=ATOL)
+
+
+def test_resident_pin_refuses_what_neither_form_takes(gpu_device):
+    dev = gpu_device
+    for (m, n, k) in [(17, 4096, 2048), (16, 4104, 4096), (16, 16384, 2304), (8, 4096, 8208)]:
+        xq, wq, xs, ws, _ = orc.make_inputs(m, n, k, 1.0, False)
+        with pytest.raises(NotImplementedError):
+            ops.fp8_gemm_rowwise(xq.to(dev), wq.to(dev), xs.to(dev), ws.to(dev), variant=PERSISTENT)
+
+
+def test_pair_kernel_ignores_what_lies_past_k(gpu_device):
+    # K = 2320 (18 whole steps and a 16-byte chunk): rows padded to 2560 bytes with codes of +-448 that must
+    # not enter any sum, neither through the partial step nor through the steps past it
+    m, n, k, ld = 16, 4096, 2320, 2560
+    xq, wq, xs, ws, b = orc.make_inputs(m, n, k, 1.0, True)
+    want = orc.dequant_matmul(xq, wq, xs, ws, b)
+    dev = gpu_device
+    a_buf = torch.full((m, ld), 0x7E, dtype=torch.uint8, device=dev)
+    b_buf = torch.full((n, ld), 0xFE, dtype=torch.uint8, device=dev)
+    a_buf[:, :k] = xq.view(torch.uint8).to(dev)
+    b_buf[:, :k] = wq.view(torch.uint8).to(dev)
+    out = ops.fp8_gemm_rowwise(a_buf.view(torch.float8_e4m3fn)[:, :k], b_buf.view(torch.float8_e4m3fn)[:, :k],
+                               xs.to(dev), ws.to(dev), bias=b.to(dev), variant=PERSISTENT)
+    torch.cuda.synchronize()
+    torch.testing.assert_close(out.cpu(), want, rtol=RTOL, atol=ATOL)
+    _check_tight(out.cpu(), xq, wq, xs, ws, b)
+
+
+@pytest.mark.parametrize("m,k", [(16, 2048), (5, 8192), (32, 4096), (19, 4096), (16, 6656), (9, 2320)])
 def test_exact_integer_case_is_bit_exact(gpu_device, m, k):
     # small integers, unit scales: every partial sum stays below 2^24, so fp32 summation is
     # exact in any order and both kernels must reproduce the float64 result bit for bit
@@ -94,11 +147,12 @@ def test_exact_integer_case_is_bit_exact(gpu_device, m, k):
         assert np.array_equal(_bits(out), want)
 
 
-def test_one_hot_positions_walk_every_k_step_and_tile(gpu_device):
-    # A[i, ka(i)] = 1 and B[j, kb(j)] = 1: C[i, j] = [ka(i) == kb(j)]. The positions walk all 64
+@pytest.mark.parametrize("n,k", [(4112, 8192), (8192, 6656), (12304, 8192), (4096, 2320)])
+def test_one_hot_positions_walk_every_k_step_and_tile(gpu_device, n, k):
+    # A[i, ka(i)] = 1 and B[j, kb(j)] = 1: C[i, j] = [ka(i) == kb(j)]. The positions walk all
     # K steps and every byte of a step, so a wrong step rotation, lane layout or tile offset
-    # shows as a misplaced one.
-    m, n, k = 16, 4112, 8192
+    # shows as a misplaced one. (N <= 8192: the pair kernel; beyond: the persistent kernel.)
+    m = 16
     ka = (np.arange(m) * 517 + 5) % k
     kb = (np.arange(n) * 131 + 2) % k
     kb[: m * 8] = np.repeat(ka, 8)  # guaranteed hits in the first tiles

@@ -23,6 +23,7 @@ VARIANT_TILED = 1
 VARIANT_SKINNY = 2
 SKINNY_ONE_TILE = 1 << 8  # skinny family: pins the one-tile-per-workgroup kernel
 SKINNY_NARROW = 2 << 8  # skinny family: pins the narrow-tile kernel (the shapes `skinny_family_takes`)
+SKINNY_RESIDENT = 4 << 8  # skinny family: pins the forms that keep A on chip (pair / persistent kernel)
 
 
 def skinny_family_takes(m: int, n: int) -> bool:

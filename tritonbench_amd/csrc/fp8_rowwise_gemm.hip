@@ -122,6 +122,17 @@ __device__ __forceinline__ uint32_t pack_out_x2(float lo, float hi, bool f16) {
   return f16 ? pack_f16x2(lo, hi) : pack_bf16x2(lo, hi);
 }
 
+// Kernel arguments live in memory and reach a wave through scalar loads that the compiler issues
+// where it first needs each value: several dependent round trips of a few hundred nanoseconds each at
+// the start of a kernel (the argument block is cold in the scalar cache at every launch). The decode
+// kernels are a few microseconds long, so they ask for everything they will use in one batch, first
+// thing (measured on the pair kernel at M=16, N=K=8192: 13.2 -> 12.6 us; whether the compiler's own
+// placement is the fast or the slow one changes with unrelated edits).
+__device__ __forceinline__ void fetch_arguments_now(const GemmParams& p) {
+  asm volatile("" ::"s"(p.a), "s"(p.b), "s"(p.a_scale), "s"(p.b_scale), "s"(p.bias), "s"(p.c), "s"(p.M), "s"(p.N), "s"(p.K),
+               "s"(p.lda), "s"(p.ldb), "s"(p.ldc), "s"(p.tiles_m), "s"(p.tiles_n), "s"(p.out_f16));
+}
+
 // ------------------------------------------------------------------------------------
 // Tile scheduler: static, no atomics (safe under graph capture).
 //
@@ -1141,6 +1152,7 @@ __global__ __launch_bounds__(KW * 64) void gemm_skinny_kernel(GemmParams p) {
   constexpr int NTILE = NTW + MT;                   // tiles per step: B tiles then A tiles
   constexpr int BUF = NTILE * TILE;                 // wave-private transpose buffer
   static_assert(NTW * MT * 1024 <= BUF, "the reduction reuses a wave's buffer for its partials");
+  fetch_arguments_now(p);
 
   extern __shared__ __attribute__((aligned(1024))) uint8_t lds[];
 
@@ -1356,6 +1368,7 @@ __global__ __launch_bounds__(kPersistWaves * 64) void gemm_skinny_persistent_ker
   constexpr int WAVES = kPersistWaves;
   constexpr int STEPS = WAVES * SPW;
   static_assert(LAG >= 1 && LAG <= SPW && SPW % LAG == 0, "the landing registers are a ring of LAG steps");
+  fetch_arguments_now(p);
   extern __shared__ __attribute__((aligned(1024))) uint8_t lds[];
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -1588,6 +1601,7 @@ __global__ __launch_bounds__(512) void gemm_narrow_kernel(GemmParams p) {
   constexpr int STA = BM * KS, STB = BN * KS;  // bytes per stage
   constexpr int LA = BM / 8, LB = BN / 8;      // wave-wide loads per wave and step (8 rows x 128 bytes each)
   static_assert((DA - 1) * LA < 64 && (DB - 1) * LB < 64, "outstanding-load counts must fit the wait instruction");
+  fetch_arguments_now(p);
   extern __shared__ __attribute__((aligned(1024))) uint8_t lds[];
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -1781,6 +1795,234 @@ __global__ __launch_bounds__(512) void gemm_narrow_kernel(GemmParams p) {
       __builtin_amdgcn_s_barrier();
     }
     __syncthreads();  // the compute waves' hand-over of their partial results
+  }
+}
+
+// ------------------------------------------------------------------------------------
+// Pair kernel: M <= 16, N a multiple of 16 up to 8192 (at most two 16-row tiles of B per CU),
+// K up to 8192 (any multiple of 16). The decode shapes proper: the whole launch is one or two
+// tiles per workgroup, so there is no steady state to reach and what counts is the order in
+// which the requests leave the CU.
+//
+// One workgroup of 16 waves per CU; wave w owns the K steps w, w+16, ... (SPW of them, those past
+// K read as zeros) as in the persistent kernel above. Differences:
+//  * A is not kept in registers: each wave copies its SPW-1 first steps of A straight from memory
+//    into LDS, already in the order the MFMA lanes read them, and reads a step's fragment from there
+//    when it multiplies; only its last step goes through the transpose buffer into registers (LDS:
+//    3 x 32 KB of A at SPW = 4, 32 KB of transpose buffers, 32 KB of partial results).
+//  * A tile's loads of B leave in one burst: step 0 of the first tile first, then A, then the rest
+//    of the first tile together with step 0 of the second; the rest of the second tile follows the
+//    first tile's reduction. A tile is 16 rows x K contiguous bytes, so a burst asks for one
+//    contiguous region, and at no time is more than one tile per CU in flight: measured cold at
+//    M=16, N=K=8192, this order 12.9 us against 13.4 us for the persistent kernel's rolling
+//    prefetch (four steps per wave in flight all the time) and 13.9 us for the same rolling
+//    prefetch with A in LDS; K = 4096 8.0 against 8.6 us, K = 2048 5.3 against 5.9, N = 4096 9.0
+//    against 9.5, M = 1 12.2 against 12.6. Everything requested at once (both tiles) takes 14.9 us.
+// All loads of B are range-checked buffer loads: a lane whose 16 bytes lie past K, and every lane of
+// a tile that does not exist, asks for an offset outside the descriptor and gets zeros without a
+// memory access, so the instruction stream is the same for every wave and the wait counts are exact.
+// ------------------------------------------------------------------------------------
+constexpr size_t pair_lds_bytes(int SPW) {
+  return (size_t)kPersistWaves * 2048 * SPW + (size_t)2 * kPersistWaves * 1024;
+}
+
+// KTAIL: K is no multiple of 2048, so some waves own steps that lie (partly) past K and their lanes need a
+// predicate per load; HAS_BIAS: a bias vector is added. Both are compile-time properties: this kernel's
+// time hangs on how fast a wave gets its burst of loads out, and the few vector instructions either adds
+// in front of the loads measured 0.3 and 0.1 us at M=16, N=K=8192.
+template <int SPW, bool VEC, bool KTAIL, bool HAS_BIAS>
+__global__ __launch_bounds__(kPersistWaves * 64) void gemm_skinny_pair_kernel(GemmParams p) {
+  constexpr int WAVES = kPersistWaves;
+  constexpr int STEPS = WAVES * SPW;
+  constexpr int A_LDS = SPW - 1;  // steps of A per wave that live in LDS
+  fetch_arguments_now(p);
+  extern __shared__ __attribute__((aligned(1024))) uint8_t lds[];
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  uint8_t* a_mine = lds + wave * (A_LDS * 2048);             // this wave's steps of A
+  uint8_t* buf = lds + WAVES * A_LDS * 2048 + wave * 2048;   // this wave's transpose buffer (one 16 x 128 B step)
+  v4f* red = (v4f*)(lds + WAVES * SPW * 2048);               // [2][WAVES][64] partial results
+
+  // this workgroup's one or two tiles (quotient and remainder of tiles by workgroups come from the host)
+  const int g = blockIdx.x;
+  const int tile0 = g * p.tiles_m + min(g, p.tiles_n);
+  const int count = p.tiles_m + (g < p.tiles_n ? 1 : 0);
+  if (count <= 0) return;
+
+  // byte offset of this wave's i-th K step inside a row; workgroups of one XCD start at different steps
+  const int base_step = (wave + 2 * (g >> 3)) % STEPS;
+  uint32_t kofs[SPW];
+#pragma unroll
+  for (int i = 0; i < SPW; ++i) {
+    int s = base_step + WAVES * i;
+    if (s >= STEPS) s -= STEPS;
+    kofs[i] = (uint32_t)__builtin_amdgcn_readfirstlane(s * kStepK);
+  }
+  const int r16 = lane & 15, g4 = lane >> 4;
+  const int ld_row = lane >> 3, ld_c = lane & 7;
+  constexpr uint32_t kOutside = 0x80000000u;  // past every extent (the host keeps extents below 2^31)
+  uint32_t b_lane[2], a_lane[2];
+  int wr_off[2];
+#pragma unroll
+  for (int h = 0; h < 2; ++h) {
+    const int r = h * 8 + ld_row;
+    wr_off[h] = r * kStepK + ((ld_c ^ swz128(r)) * kChunk);
+    b_lane[h] = (uint32_t)r * (uint32_t)p.ldb + ld_c * kChunk;
+    // the direct-to-LDS copy puts lane l at position l of a 1 KB half step (8 rows x 128 bytes): the lane
+    // asks for the chunk whose swizzled place that is; rows past M repeat the last one
+    a_lane[h] = (uint32_t)min(r, p.M - 1) * (uint32_t)p.lda + (uint32_t)((ld_c ^ swz128(r)) * kChunk);
+  }
+  // the lane's chunk of a step lies inside K? (only the last step of a K that is no multiple of 128 cuts lanes off)
+  auto in_k = [&](uint32_t step_off, int chunk) { return !KTAIL || step_off + (uint32_t)(chunk * kChunk) < (uint32_t)p.K; };
+  const int rd0 = r16 * kStepK + (((2 * g4) ^ swz128(r16)) * kChunk);
+  const int rd1 = r16 * kStepK + (((2 * g4 + 1) ^ swz128(r16)) * kChunk);
+
+  const uint32_t tile_pitch = 16u * (uint32_t)p.ldb;
+  const uintptr_t bb = reinterpret_cast<uintptr_t>(p.b) + (size_t)tile0 * tile_pitch;
+  const uint8_t* b_base = reinterpret_cast<const uint8_t*>(
+      ((uintptr_t)(uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)(bb >> 32)) << 32) |
+      (uintptr_t)(uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)bb));
+  const __amdgpu_buffer_rsrc_t rb = __builtin_amdgcn_make_buffer_rsrc(
+      const_cast<uint8_t*>(b_base), 0, (int)((uint32_t)count * tile_pitch), 0x00020000);
+  const __amdgpu_buffer_rsrc_t ra = __builtin_amdgcn_make_buffer_rsrc(
+      const_cast<uint8_t*>(p.a), 0, (int)((uint32_t)p.M * (uint32_t)p.lda), 0x00020000);
+
+  v4i land[2][SPW][2];
+  auto fetch = [&](int t, int i) {
+    const uint32_t so = (uint32_t)t * tile_pitch + kofs[i];
+    const bool ok = t < count && in_k(kofs[i], ld_c);
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+#if defined(__HIP_DEVICE_COMPILE__)
+      land[t][i][h] = __builtin_bit_cast(v4i, __builtin_amdgcn_raw_buffer_load_b128(rb, (int)(ok ? b_lane[h] : kOutside), (int)so, 2));
+#else
+      land[t][i][h] = (v4i){0, 0, 0, 0};
+#endif
+    }
+  };
+  fetch(0, 0);  // the first rows of B are asked for before anything else: they come from HBM
+  __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+  for (int i = 0; i < SPW; ++i) {
+    uint8_t* dst = i < A_LDS ? a_mine + i * 2048 : buf;
+    // (the chunk a lane fetches for LDS position ld_c of row r is ld_c ^ swz128(r))
+#pragma unroll
+    for (int h = 0; h < 2; ++h)
+      load_chunk_to_lds<false>(ra, dst + h * 1024, in_k(kofs[i], ld_c ^ swz128(h * 8 + ld_row)) ? a_lane[h] : kOutside, kofs[i]);
+  }
+  __builtin_amdgcn_sched_barrier(0);
+  // Wave j finishes tile j: lane (m = lane % 16, quad lane / 16) owns C[m, 16*tile + 4*(lane/16) .. +3] (waves
+  // without a result read the run's last tile and drop it). Its scales and bias come from memory nobody has
+  // touched yet, so they are asked for here, while the wave waits for A anyway - but the wait below must not
+  // include them (it holds the burst back: 0.3 us at M=16, N=K=8192), so it has to know how many load
+  // instructions they are. With aligned vectors that is exact: one buffer load each through descriptors of
+  // their own (nothing the compiler could merge or split). The unaligned form asks behind the burst instead.
+  const int fin_n = (tile0 + min(wave, count - 1)) * 16 + 4 * g4;
+  float fin_sa = 0.f, sb_raw[4] = {0.f, 0.f, 0.f, 0.f};
+  uint16_t bias_raw[4] = {0, 0, 0, 0};
+  if constexpr (VEC) {
+#if defined(__HIP_DEVICE_COMPILE__)
+    const __amdgpu_buffer_rsrc_t rsa = __builtin_amdgcn_make_buffer_rsrc(const_cast<float*>(p.a_scale), 0, p.M * 4, 0x00020000);
+    const __amdgpu_buffer_rsrc_t rsb = __builtin_amdgcn_make_buffer_rsrc(const_cast<float*>(p.b_scale), 0, p.N * 4, 0x00020000);
+    fin_sa = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(rsa, min(r16, p.M - 1) * 4, 0, 0));
+    const v4f s4 = load_f32x4_checked(rsb, (uint32_t)fin_n * 4u);
+#pragma unroll
+    for (int x = 0; x < 4; ++x) sb_raw[x] = s4[x];
+    if (HAS_BIAS) {
+      const __amdgpu_buffer_rsrc_t rbias = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint16_t*>(p.bias), 0, p.N * 2, 0x00020000);
+      const us4 b4 = load_u16x4_checked(rbias, (uint32_t)fin_n * 2u);
+#pragma unroll
+      for (int x = 0; x < 4; ++x) bias_raw[x] = b4[x];
+    }
+#endif
+    __builtin_amdgcn_sched_barrier(0);
+    // A has landed once everything in front of those two or three loads has (loads return in order)
+    wait_loads<2 + (HAS_BIAS ? 1 : 0)>();
+  } else {
+    wait_loads<0>();
+  }
+  v8i fa_last;
+  {
+    const v4i lo = *(const v4i*)(buf + rd0);
+    const v4i hi = *(const v4i*)(buf + rd1);
+    fa_last = (v8i){lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+    __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0): in registers before the buffer is written again
+  }
+  __builtin_amdgcn_sched_barrier(0);
+
+  auto consume = [&](int t, int i, v4f& acc) {
+    *(v4i*)(buf + wr_off[0]) = land[t][i][0];
+    *(v4i*)(buf + wr_off[1]) = land[t][i][1];
+    const v4i lo = *(const v4i*)(buf + rd0);
+    const v4i hi = *(const v4i*)(buf + rd1);
+    const v8i fb = (v8i){lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+    v8i fa = fa_last;
+    if (i < A_LDS) {
+      const v4i alo = *(const v4i*)(a_mine + i * 2048 + rd0);
+      const v4i ahi = *(const v4i*)(a_mine + i * 2048 + rd1);
+      fa = (v8i){alo[0], alo[1], alo[2], alo[3], ahi[0], ahi[1], ahi[2], ahi[3]};
+    }
+    acc = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(fb, fa, acc, 0, 0, 0, 0, 0, 0);
+  };
+  // tile 0: the rest of its loads in one burst, the first step of tile 1 behind them
+#pragma unroll
+  for (int i = 1; i < SPW; ++i) fetch(0, i);
+  fetch(1, 0);
+  __builtin_amdgcn_sched_barrier(0);
+  if constexpr (!VEC) {  // (element by element: a count the compiler may change, so behind the burst)
+    fin_sa = p.a_scale[min(r16, p.M - 1)];
+#pragma unroll
+    for (int x = 0; x < 4; ++x) {
+      sb_raw[x] = p.b_scale[fin_n + x];
+      if (HAS_BIAS) bias_raw[x] = p.bias[fin_n + x];
+    }
+  }
+  __builtin_amdgcn_sched_barrier(0);
+  // the 16 partial results of tile j meet in LDS (one area per tile); wave j adds them in wave order and stores
+  auto finish = [&](int j, const v4f& acc) {
+    v4f* area = red + j * (WAVES * 64);
+    area[wave * 64 + lane] = acc;
+    __syncthreads();
+    if (wave == j) {
+      const v4f* part = area + lane;
+      v4f sum = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll 1
+      for (int w0 = 0; w0 < WAVES; w0 += 8) {  // eight partials in flight at a time
+#pragma unroll
+        for (int w = 0; w < 8; ++w) sum += part[(w0 + w) * 64];
+      }
+      if (r16 < p.M) {
+        float r[4];
+#pragma unroll
+        for (int x = 0; x < 4; ++x)
+          r[x] = HAS_BIAS ? __builtin_fmaf(sum[x] * fin_sa, sb_raw[x], bf16_to_f32(bias_raw[x])) : sum[x] * fin_sa * sb_raw[x];
+        const uint32_t lo = pack_out_x2(r[0], r[1], p.out_f16), hi = pack_out_x2(r[2], r[3], p.out_f16);
+        uint16_t* dst = p.c + (size_t)r16 * p.ldc + (tile0 + j) * 16 + 4 * g4;
+        if (VEC) {
+          *(v2u*)dst = (v2u){lo, hi};
+        } else {
+          dst[0] = (uint16_t)lo; dst[1] = (uint16_t)(lo >> 16);
+          dst[2] = (uint16_t)hi; dst[3] = (uint16_t)(hi >> 16);
+        }
+      }
+    }
+  };
+
+  v4f acc0 = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+  for (int i = 0; i < SPW; ++i) consume(0, i, acc0);
+  __builtin_amdgcn_sched_barrier(0);
+  finish(0, acc0);
+  __builtin_amdgcn_sched_barrier(0);
+  // tile 1 (loads that ask for nothing when there is none: the instruction stream stays the same)
+#pragma unroll
+  for (int i = 1; i < SPW; ++i) fetch(1, i);
+  __builtin_amdgcn_sched_barrier(0);
+  if (count > 1) {
+    v4f acc1 = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int i = 0; i < SPW; ++i) consume(1, i, acc1);
+    finish(1, acc1);
   }
 }
 
@@ -2238,6 +2480,10 @@ constexpr TileConfig kTileConfigs[kNumTileConfigs] = {
 // four blocks the register budget leaves one workgroup per CU, and a last round of workgroups
 // that fills only part of the CUs streams at that fraction of the rate.
 inline bool persistent_skinny_fits(int64_t M, int64_t N, int64_t K);
+// The pair kernel: up to 16 rows of A, at most two 16-row tiles of B per CU, K that fits the LDS.
+inline bool pair_skinny_fits(int64_t M, int64_t N, int64_t K) {
+  return M <= 16 && N % 16 == 0 && N <= 2 * 16 * kNumCu && K <= 4 * kPersistWaves * kStepK;
+}
 // The narrow-tile kernel. With all rows in one workgroup (M <= 64) its cost is one round of workgroups per
 // 256 tiles (measured at N = 8192, cold: 9.8 / 14.3 / 43.0 us for K = 4096 / 8192 / 28672 with up to
 // 32 rows of A, 17.1-17.9 / 49.9 us for K = 8192 / 28672 with up to 64).
@@ -2304,6 +2550,8 @@ inline float narrow_cost_us(int64_t M, int64_t N, int64_t K) {
 inline float skinny_streaming_cost_us(int64_t M, int64_t N, int64_t K) {
   // the persistent form (measured: 12.7 us at N=K=8192, 71 us at N=57344)
   // (two blocks of A, K = 4096: 9.9 us at N=8192)
+  // the pair kernel (measured cold: 12.9 us at N=K=8192, 8.0 at K=4096, 5.3 at K=2048; 9.0 at 4096 x 8192, one tile per CU)
+  if (pair_skinny_fits(M, N, K)) return (N <= 16 * kNumCu ? 4.0f : 2.9f) + (float)N * (float)K / 6.7e6f;
   if (persistent_skinny_fits(M, N, K)) return 3.0f + (float)N * (float)K / (M <= 16 ? 6.9e6f : 4.9e6f);
   static const float rate[4] = {6.0e6f, 4.5e6f, 3.44e6f, 3.6e6f};
   const int blocks = (int)((M + 15) / 16);
@@ -2614,6 +2862,42 @@ int launch_skinny_persistent(const GemmParams& p, hipStream_t stream) {
   return MI355X_FP8_OK;
 }
 
+template <int SPW, bool VEC, bool KTAIL, bool HAS_BIAS>
+int launch_skinny_pair(const GemmParams& p, hipStream_t stream) {
+  constexpr size_t lds_bytes = pair_lds_bytes(SPW);
+  static_assert(lds_bytes <= 160 * 1024, "A's steps, the transpose buffers and the partial results must fit the LDS");
+  constexpr auto kern = gemm_skinny_pair_kernel<SPW, VEC, KTAIL, HAS_BIAS>;
+  (void)LdsLimit<kern, lds_bytes>::registered;
+  if (const int st = ready_device()) return st;
+  const long ntiles = p.N / 16;
+  const unsigned grid = (unsigned)(ntiles < kNumCu ? ntiles : kNumCu);
+  GemmParams q = p;
+  q.tiles_m = (int)(ntiles / grid);  // tiles per workgroup ...
+  q.tiles_n = (int)(ntiles % grid);  // ... and how many workgroups take one more
+  hipLaunchKernelGGL(kern, dim3(grid), dim3(kPersistWaves * 64), lds_bytes, stream, q);
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess) return fail(MI355X_FP8_ELAUNCH, "pair skinny kernel launch: %s", hipGetErrorString(e));
+  return MI355X_FP8_OK;
+}
+
+template <bool VEC, bool KTAIL, bool HAS_BIAS>
+int launch_skinny_pair_steps(const GemmParams& p, hipStream_t s) {
+  const int steps = (p.K + kStepK - 1) / kStepK;
+  const int spw = (steps + kPersistWaves - 1) / kPersistWaves;
+  switch (spw) {
+    case 1: return launch_skinny_pair<1, VEC, KTAIL, HAS_BIAS>(p, s);
+    case 2: return launch_skinny_pair<2, VEC, KTAIL, HAS_BIAS>(p, s);
+    case 3: return launch_skinny_pair<3, VEC, KTAIL, HAS_BIAS>(p, s);
+    default: return launch_skinny_pair<4, VEC, KTAIL, HAS_BIAS>(p, s);
+  }
+}
+template <bool VEC>
+int launch_skinny_pair_form(const GemmParams& p, hipStream_t s) {
+  const bool ktail = p.K % (kPersistWaves * kStepK) != 0;
+  if (p.bias) return ktail ? launch_skinny_pair_steps<VEC, true, true>(p, s) : launch_skinny_pair_steps<VEC, false, true>(p, s);
+  return ktail ? launch_skinny_pair_steps<VEC, true, false>(p, s) : launch_skinny_pair_steps<VEC, false, false>(p, s);
+}
+
 template <bool VEC>
 int launch_skinny_persistent_steps(const GemmParams& p, hipStream_t s) {
   const int spw = p.K / (kPersistWaves * kStepK);
@@ -2815,12 +3099,19 @@ int run_gemm(const void* a, const void* b, const float* a_scale, const float* b_
           return fail(MI355X_FP8_ENOTSUP, "the one-tile-per-workgroup form takes M <= %d (got M=%lld)", kSkinnyMaxM, (long long)M);
         return launch_narrow_for(p, s);
       }
-      if (!(plan_bits & MI355X_FP8_SKINNY_ONE_TILE) && narrow_preferred(M, N, K)) return launch_narrow_for(p, s);
-      if (persistent_skinny_fits(M, N, K) && !(plan_bits & MI355X_FP8_SKINNY_ONE_TILE)) {
+      if (!(plan_bits & (MI355X_FP8_SKINNY_ONE_TILE | MI355X_FP8_SKINNY_RESIDENT)) && narrow_preferred(M, N, K))
+        return launch_narrow_for(p, s);
+      if ((plan_bits & MI355X_FP8_SKINNY_RESIDENT) && !pair_skinny_fits(M, N, K) && !persistent_skinny_fits(M, N, K))
+        return fail(MI355X_FP8_ENOTSUP, "neither form that keeps A on chip takes %lldx%lldx%lld", (long long)M, (long long)N, (long long)K);
+      if ((pair_skinny_fits(M, N, K) || persistent_skinny_fits(M, N, K)) && !(plan_bits & MI355X_FP8_SKINNY_ONE_TILE)) {
         // 16-byte loads of b_scale, 8-byte loads of bias and 8-byte stores of C when everything is aligned for them
         const bool vec = (reinterpret_cast<uintptr_t>(b_scale) & 15) == 0 && (reinterpret_cast<uintptr_t>(bias) & 7) == 0 &&
                          (reinterpret_cast<uintptr_t>(c) & 7) == 0 && (ldc & 3) == 0;
-        return vec ? launch_skinny_persistent_steps<true>(p, s) : launch_skinny_persistent_steps<false>(p, s);
+        // (the pair kernel addresses a workgroup's rows of B with 32-bit offsets below 2^31)
+        if (pair_skinny_fits(M, N, K) && ldb * 32 <= (int64_t)INT32_MAX)
+          return vec ? launch_skinny_pair_form<true>(p, s) : launch_skinny_pair_form<false>(p, s);
+        if (persistent_skinny_fits(M, N, K))
+          return vec ? launch_skinny_persistent_steps<true>(p, s) : launch_skinny_persistent_steps<false>(p, s);
       }
       if (M <= 16) return launch_skinny<1, 1, 4, 8>(p, s);
       if (M <= 32) return launch_skinny<2, 1, 2, 8>(p, s);
