@@ -423,6 +423,9 @@ def profile_kernel(which, dev):
     if which == "tiled":
         sets, wsp = make_sets(8192, make_weights(8192, 8192, 1.0, False, dev, 1), 1.0, dev)
         fig = figures(8192, 8192, 8192, False, time_steps(sets, wsp, 20, 5))
+    elif which == "tiled_cold":  # (five operand sets: A and B of a call come from HBM, not from the memory-side cache)
+        sets, wsp = make_sets(8192, make_weights(8192, 8192, 1.0, False, dev, 5), 1.0, dev)
+        fig = figures(8192, 8192, 8192, False, time_steps(sets, wsp, 20, 5))
     elif which == "skinny":
         sets, wsp = make_sets(16, make_weights(8192, 8192, 1.0, False, dev, 10), 1.0, dev)
         fig = figures(16, 8192, 8192, False, time_steps(sets, wsp, 40, 10))
@@ -466,7 +469,7 @@ def main():
     ap.add_argument("--no-extra", action="store_true", help="headline workload only")
     ap.add_argument("--vendor", action="store_true",
                     help="also time torch._scaled_mm (hipBLASLt, row-wise scales) on every GEMM row's operands")
-    ap.add_argument("--profile-kernel", choices=["tiled", "skinny", "quantise", "fused", "grouped", "decode32", "decode128", "decode128_n10240", "decode128_n57344", "ragged"],
+    ap.add_argument("--profile-kernel", choices=["tiled", "tiled_cold", "skinny", "quantise", "fused", "grouped", "decode32", "decode128", "decode128_n10240", "decode128_n57344", "ragged"],
                     help="run only that kernel's workload a few times (for rocprofv3 counter passes) and print its figures")
     args = ap.parse_args()
     global VENDOR

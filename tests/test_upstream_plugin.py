@@ -133,6 +133,99 @@ def test_registered_backend_returns_a_capturable_callable(gpu_device, monkeypatc
     torch.testing.assert_close(res.cpu(), want, rtol=1e-2, atol=1e-2)
 
 
+SIBLINGS = {
+    # operator name -> (registrar, backend names, parameters of the first backend as upstream declares them)
+    "fp8_gemm_rowwise_grouped": ("register_grouped", ["_hip_mi355x"], ["self", "group_A", "group_B", "m_sizes", "a_scale", "b_scale"]),
+    "fp8_gemm_blockwise": ("register_blockwise", ["_hip_mi355x"], ["self", "xq", "wq", "x_scale", "w_scale"]),
+    "fp8_gemm": ("register_tensorwise", ["_hip_mi355x"], ["self", "a", "b"]),
+    "fp8_fused_quant_gemm_rowwise": ("register_fused_quant", ["rms_norm_fused_hip_mi355x", "silu_mul_fused_hip_mi355x"],
+                                     ["self", "x1", "x2", "wq", "w_scale", "wd"]),
+}
+
+
+@pytest.mark.parametrize("operator_name", sorted(SIBLINGS))
+def test_sibling_operators_register_under_their_own_names(monkeypatch, operator_name):
+    """fp8_gemm_rowwise_grouped/operator.py:400-455, fp8_gemm_blockwise/operator.py:139-145,
+    fp8_gemm/fp8_gemm.py:87-101, fp8_fused_quant_gemm_rowwise/operator.py:86-131: the backend
+    methods take exactly the example inputs those operators yield."""
+    mod, calls = _install_upstream_stub(monkeypatch)
+    from tritonbench_amd import upstream_plugin
+
+    registrar, names, params = SIBLINGS[operator_name]
+
+    class FakeOperator:
+        pass
+
+    upstream_plugin.register_for(operator_name, FakeOperator)
+    assert [c["func_name"] for c in calls] == names
+    assert all(c["operator_name"] == operator_name and not c["baseline"] for c in calls)
+    assert list(mod.REGISTERED_BENCHMARKS) == [operator_name]
+    for name in names:
+        assert list(inspect.signature(getattr(FakeOperator, name)).parameters) == params
+    assert upstream_plugin.REGISTRARS[operator_name] is getattr(upstream_plugin, registrar)
+    with pytest.raises(KeyError, match="no MI355X backend"):
+        upstream_plugin.register_for("addmm", FakeOperator)
+
+
+@pytest.mark.gpu
+def test_sibling_backends_match_the_oracle(gpu_device, monkeypatch):
+    """Each registered sibling backend, called the way upstream calls it, against the CPU oracle."""
+    _install_upstream_stub(monkeypatch)
+    from oracle import fp8_rowwise as orc
+    from tritonbench_amd import upstream_plugin
+
+    dev = gpu_device
+
+    def make(name, **attrs):
+        cls = type("FakeOperator", (), dict(attrs))
+        upstream_plugin.register_for(name, cls)
+        return cls()
+
+    # grouped: G groups of the same N, K; sizes on the device
+    g, n, k = 3, 256, 512
+    sizes = [70, 0, 130]
+    xq, _, xs, _, _ = orc.make_inputs(sum(sizes), 16, k, 1.0, False)
+    _, wq, _, ws, _ = orc.make_inputs(16, g * n, k, 1.0, False)
+    m_sizes = torch.tensor(sizes, dtype=torch.int32, device=dev)
+    fn = make("fp8_gemm_rowwise_grouped")._hip_mi355x(xq.to(dev), wq.to(dev), m_sizes, xs.to(dev), ws.to(dev))
+    got = fn().cpu()
+    start = 0
+    for gi, mg in enumerate(sizes):
+        want = orc.dequant_matmul(xq[start:start + mg], wq[gi * n:(gi + 1) * n], xs[start:start + mg], ws[gi * n:(gi + 1) * n], None)
+        torch.testing.assert_close(got[start:start + mg], want, rtol=1e-2, atol=1e-2)
+        start += mg
+
+    # tensor-wise: b is [K, N] column-major; both scale conventions
+    a = torch.randn(200, 384).to(torch.float8_e4m3fn)
+    b = torch.randn(384, 272).to(torch.float8_e4m3fn).T.contiguous().T
+    want = a.to(torch.float32) @ b.to(torch.float32)
+    for rowwise, dtype in ((False, torch.float16), (True, torch.bfloat16)):
+        op = make("fp8_gemm", extra_args=types.SimpleNamespace(scaling_rowwise=rowwise))
+        got = op._hip_mi355x(a.to(dev), b.to(dev))()
+        assert got.dtype == dtype
+        torch.testing.assert_close(got.cpu().to(torch.float32), want.to(dtype).to(torch.float32), rtol=1e-2, atol=1e-2)
+
+    # block-wise: one scale per 128 x 128 block of either operand
+    xq, wq, x_scale, w_scale = orc.make_blockwise_inputs(192, 256, 512)
+    got = make("fp8_gemm_blockwise")._hip_mi355x(xq.to(dev), wq.to(dev), x_scale.to(dev), w_scale.to(dev))().cpu()
+    torch.testing.assert_close(got, orc.blockwise_dequant_matmul(xq, wq, x_scale, w_scale), rtol=1e-2, atol=1e-2)
+
+    # fused front ends: same result as the separate steps of this package
+    from tritonbench_amd import ops
+
+    x1 = torch.randn(64, 512, dtype=torch.bfloat16, device=dev)
+    x2 = torch.randn(64, 512, dtype=torch.bfloat16, device=dev)
+    wdn = torch.randn(512, dtype=torch.bfloat16, device=dev)
+    wq2, w_scale2 = ops.fp8_row_quantize(torch.randn(128, 512, dtype=torch.bfloat16, device=dev))
+    op = make("fp8_fused_quant_gemm_rowwise")
+    got = op.rms_norm_fused_hip_mi355x(x1, x2, wq2, w_scale2, wdn)()
+    q, s = ops.rms_norm_fp8_rowwise_quant(x1, wdn, 1e-5)
+    assert torch.equal(got, ops.fp8_gemm_rowwise(q, wq2, s, w_scale2))
+    got = op.silu_mul_fused_hip_mi355x(x1, x2, wq2, w_scale2, wdn)()
+    q, s = ops.silu_mul_fp8_rowwise_quant(x1, x2)
+    assert torch.equal(got, ops.fp8_gemm_rowwise(q, wq2, s, w_scale2))
+
+
 @pytest.mark.gpu
 @pytest.mark.parametrize("extra", [["--m", "1000", "--n", "3000", "--k", "4112", "--bias"], ["--m", "16", "--n", "8192", "--k", "2048"]])
 def test_harness_accuracy_tflops_gbps_on_the_hip_backend(gpu_device, extra):

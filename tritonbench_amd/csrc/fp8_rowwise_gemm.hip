@@ -132,6 +132,11 @@ __device__ __forceinline__ void fetch_arguments_now(const GemmParams& p) {
   asm volatile("" ::"s"(p.a), "s"(p.b), "s"(p.a_scale), "s"(p.b_scale), "s"(p.bias), "s"(p.c), "s"(p.M), "s"(p.N), "s"(p.K),
                "s"(p.lda), "s"(p.ldb), "s"(p.ldc), "s"(p.tiles_m), "s"(p.tiles_n), "s"(p.out_f16));
 }
+// the same for what only the tiled kernel and its second pass read
+__device__ __forceinline__ void fetch_tiled_arguments_now(const GemmParams& p) {
+  asm volatile("" ::"s"(p.splits), "s"(p.steps_per_split), "s"(p.partial), "s"(p.m_sizes), "s"(p.groups), "s"(p.div_tiles_mul),
+               "s"(p.div_tiles_shift), "s"(p.div_group_mul), "s"(p.div_group_shift), "s"(p.stamps));
+}
 
 // ------------------------------------------------------------------------------------
 // Tile scheduler: static, no atomics (safe under graph capture).
@@ -342,6 +347,8 @@ void gemm_tiled_kernel(GemmParams p) {
   static_assert(WTM % 32 == 0 && WTN % 32 == 0, "wave tile must be a multiple of 32x32");
   static_assert(DIST * (A_GROUPS + B_GROUPS) < 64, "outstanding-load count must fit the vmcnt field");
 
+  fetch_arguments_now(p);
+  fetch_tiled_arguments_now(p);
   extern __shared__ __attribute__((aligned(1024))) uint8_t lds[];
 
   // (diagnostic launches only: the shader clock and the constant 100 MHz clock at this workgroup's start)
@@ -1085,6 +1092,8 @@ void gemm_tiled_kernel(GemmParams p) {
 // depend on scheduling), applies the scales and the bias and rounds to bf16. One thread per
 // 4 consecutive columns.
 __global__ __launch_bounds__(256) void splitk_finalize_kernel(GemmParams p) {
+  fetch_arguments_now(p);
+  fetch_tiled_arguments_now(p);
   const long quads_per_row = (p.N + 3) / 4;
   const long idx = (long)blockIdx.x * 256 + threadIdx.x;
   if (idx >= quads_per_row * p.M) return;
@@ -2536,7 +2545,9 @@ inline float narrow_cost_us(int64_t M, int64_t N, int64_t K) {
   }
   // (K = 28672, N = 10240, M = 32: 58.7 us, a lower rate than the shorter rows reach)
   if (narrow_is_wide(N))
-    return M <= 32 ? 4.0f + (float)N * (float)K / (K > 16384 ? 5.0e6f : 6.3e6f) : 8.0f + (float)N * (float)K / (K > 16384 ? 5.5e6f : 7.0e6f);
+    // (four 512-byte steps, K = 2048: 7.4 us at 4 x 13312)
+    return M <= 32 ? (K <= 2048 ? 3.0f : 4.0f) + (float)N * (float)K / (K > 16384 ? 5.0e6f : 6.3e6f)
+                   : 8.0f + (float)N * (float)K / (K > 16384 ? 5.5e6f : 7.0e6f);
   const long tiles = (N + 31) / 32;
   const long rounds = (tiles + kNumCu - 1) / kNumCu;
   // per 1024 bytes of K: what the CUs at work can pull from L2, or, with most of them at work and up to 32
@@ -2550,9 +2561,10 @@ inline float narrow_cost_us(int64_t M, int64_t N, int64_t K) {
 inline float skinny_streaming_cost_us(int64_t M, int64_t N, int64_t K) {
   // the persistent form (measured: 12.7 us at N=K=8192, 71 us at N=57344)
   // (two blocks of A, K = 4096: 9.9 us at N=8192)
-  // the pair kernel (measured cold: 12.9 us at N=K=8192, 8.0 at K=4096, 5.3 at K=2048; 9.0 at 4096 x 8192, one tile per CU)
-  if (pair_skinny_fits(M, N, K)) return (N <= 16 * kNumCu ? 4.0f : 2.9f) + (float)N * (float)K / 6.7e6f;
-  if (persistent_skinny_fits(M, N, K)) return 3.0f + (float)N * (float)K / (M <= 16 ? 6.9e6f : 4.9e6f);
+  // the pair kernel (measured cold: 12.75 us at N=K=8192, 7.9 at K=4096, 5.4 at K=2048; 8.7 at 4096 x 8192, one tile per CU)
+  if (pair_skinny_fits(M, N, K)) return (N <= 16 * kNumCu ? 3.75f : 2.75f) + (float)N * (float)K / 6.7e6f;
+  // (one step per wave, K = 2048: a tile is over before the next one's rows have arrived; 4 x 13312 x 2048 8.2 us)
+  if (persistent_skinny_fits(M, N, K)) return (K <= 2048 ? 4.2f : 3.0f) + (float)N * (float)K / (M <= 16 ? 6.9e6f : 4.9e6f);
   static const float rate[4] = {6.0e6f, 4.5e6f, 3.44e6f, 3.6e6f};
   const int blocks = (int)((M + 15) / 16);
   const int b = blocks < 1 ? 0 : blocks > 4 ? 3 : blocks - 1;
