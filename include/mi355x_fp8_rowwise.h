@@ -60,7 +60,9 @@ extern "C" {
  * field = chosen by the library from the shape). Tile configurations: 0 = 256x256 tiles,
  * one workgroup per CU; 1 = 128x128 tiles, two workgroups per CU; 2 = 256x128 tiles
  * (256 rows of A, 128 rows of B), one workgroup per CU; 3 = 64x256, 4 = 128x256 and 5 = 192x256 tiles, one
- * workgroup per CU (none of the three available in the grouped form). With a split-K factor
+ * workgroup per CU; 6 = 128x128 tiles with a deeper ring of loads in flight, one workgroup per CU
+ * (chosen by the library only for launches of at most 256 work items and not split; pinned, it
+ * runs any shape). Configurations 3 to 6 are not available in the grouped form. With a split-K factor
  * S > 1 every tile's K range is cut into S parts that run as separate work items; they
  * leave fp32 partial sums in the workspace (S*M*N*4 bytes) and a second kernel adds them
  * in a fixed order, so results do not depend on scheduling. A split factor larger than the
@@ -85,7 +87,7 @@ extern "C" {
 #define MI355X_FP8_SKINNY_RESIDENT      (4 << 8)
 #define MI355X_FP8_TILED_CONFIG(cfg)    ((((cfg) + 1) & 0xff) << 8)
 #define MI355X_FP8_TILED_SPLITS(s)      (((s) & 0xff) << 16)
-#define MI355X_FP8_NUM_TILE_CONFIGS     6
+#define MI355X_FP8_NUM_TILE_CONFIGS     7
 #define MI355X_FP8_NUM_GROUPED_TILE_CONFIGS 3
 
 /* Source element types accepted by the quantiser. */

@@ -32,7 +32,10 @@ SHAPES = [(32, 8192, 8192, False), (64, 8192, 8192, False), (128, 8192, 8192, Fa
           # first is the shape of its stored run configuration
           (16, 13312, 13312, False), (1, 8192, 16384, False), (4, 13312, 2048, False), (8, 8192, 6656, False),
           (16, 4096, 6656, False), (32, 2304, 16384, False), (32, 8192, 13312, False), (64, 13312, 2048, False),
-          (128, 2304, 6656, False), (128, 8192, 2304, False)]
+          (128, 2304, 6656, False), (128, 8192, 2304, False),
+          # at most one 128x128 work item per CU: the deep-ring configuration, unsplit and split
+          (1024, 2048, 4096, False), (2048, 2048, 2048, False), (1024, 1024, 8192, False), (1024, 2048, 16384, False),
+          (768, 2048, 2048, False)]
 
 
 def _time_us(dev, m, n, k, bias, variant, sets):

@@ -34,7 +34,7 @@ def skinny_family_takes(m: int, n: int) -> bool:
         return True
     return m <= 256 and -(-m // 64) * ((-(-n // 64) + 7) // 8 * 8) <= 256
 
-NUM_TILE_CONFIGS = 6
+NUM_TILE_CONFIGS = 7
 NOALLOC_SCRATCH_BYTES = 64 << 20
 STAMP_ENTRIES = 2048
 NUM_GROUPED_TILE_CONFIGS = 3

@@ -2466,7 +2466,8 @@ struct TileConfig {
   float stream_bytes_per_us;  // operand bytes per microsecond the configuration can stream from HBM
   float wg_stream_share;      // what one workgroup can stream, in units of 1/256 of that rate
 };
-constexpr int kNumTileConfigs = 6;
+constexpr int kNumTileConfigs = 7;
+constexpr int kDeepSmallConfig = 6;  // 128x128 tiles with three steps in flight, one workgroup per CU
 constexpr int kNumGroupedTileConfigs = 3;  // the grouped form uses the first three
 // Measured on MI355X with normally distributed operands (clock under sustained MFMA load).
 constexpr TileConfig kTileConfigs[kNumTileConfigs] = {
@@ -2481,6 +2482,16 @@ constexpr TileConfig kTileConfigs[kNumTileConfigs] = {
     // 1024 x 10240 x 8192 73.3 us with 240 tiles, 2048 x 10240 x 8192 135.4 us with 440)
     // (one tile row against a wide panel: 192 x 57344 x 8192 89.2 us)
     {192, 256, tiled_wgs_per_cu(192, 256), 1.00f, 1.00f, 9.0f, 4.9e6f, 1.42f},
+    // 128x128 tiles with loads three steps ahead (112 KB of LDS: one workgroup per CU), for launches of at most
+    // one workgroup per CU, where a CU has one wave per SIMD and nothing but the depth of the ring to cover
+    // the memory latency with. Operands from HBM, against the two-step form: 1024 x 2048 x 4096 25.4 -> 20.4 us
+    // with 128 tiles, 512 x 4096 x 4096 25.6 -> 21.1, 1536 x 1536 x 4096 25.4 -> 20.6, 2048 x 2048 x 4096 27.2 ->
+    // 23.0 with 256, 2048^3 15.9 -> 14.4; split (work items still at most one per CU): 1024 x 2048 x 8192 36.1 ->
+    // 31.3 in two, 1024 x 2048 x 16384 67.3 -> 48.9 in two, 1024 x 1024 x 8192 36.3 -> 26.5 in two -> 23.0 in four.
+    // Operands from the memory-side cache: 0.31 us per step instead of 0.49 (1024 x 2048 x 8192 29.1 -> 24.6).
+    // A ring one step deeper measured the same. The step time is the one with operands from HBM and half the
+    // CUs at work; plan_cost_us adds what a fuller chip costs.
+    {128, 128, 1, 0.49f, 0.49f, 4.8f, 4.4e6f, 1.18f},
 };
 
 // The skinny kernel's run time for comparison with the tiled plans at M <= 64: a fixed part
@@ -2626,6 +2637,12 @@ inline float plan_cost_us(int64_t M, int64_t N, int64_t K, int config, int split
   const long full_rounds = items / slots, rest = items % slots;
   float t = full_rounds * (sps * c.us_per_step + c.us_per_item);
   if (rest) t += sps * (rest <= kNumCu ? c.us_per_step_alone : c.us_per_step) + c.us_per_item;
+  // (the deep 128x128 form is for one round only; beyond 128 workgroups its steps slow down with the chip's
+  // clock and the shared L2: 0.49 us with 128, 0.58 with 256)
+  if (config == kDeepSmallConfig) {
+    if (items > kNumCu) return 1e30f;
+    if (items > kNumCu / 2) t += sps * 0.09f * (float)(items - kNumCu / 2) / (float)(kNumCu / 2);
+  }
   // (one or two tile rows, one for 256x256 tiles: B is fetched with the streaming policy, which is worth 8 % or more)
   const bool streams_b = (M + c.bm - 1) / c.bm <= stream_tile_rows(c.bm, c.bn);
   // (fewer work items than CUs: the busy CUs cannot make up for the idle ones beyond their share)
@@ -2638,7 +2655,7 @@ inline float plan_cost_us(int64_t M, int64_t N, int64_t K, int config, int split
   // has to take in beside its rows of B shrinks with them: 64 x 28672 x 8192 unsplit 42.4 us = 6.3 MB/us)
   const float rows_a = (float)M / (float)((M + c.bm - 1) / c.bm);
   // (not below 33 rows: there the estimate would undercut the streaming kernels, which measure 25 % ahead)
-  const float fill = config == 1 && M > 32 ? fmaxf(0.75f, (rows_a + (float)c.bn) / (float)(c.bm + c.bn)) : 1.0f;
+  const float fill = (config == 1 || config == kDeepSmallConfig) && M > 32 ? fmaxf(0.75f, (rows_a + (float)c.bn) / (float)(c.bm + c.bn)) : 1.0f;
   const float stream = ((float)M * (float)K + (float)N * (float)K) * fill / (c.stream_bytes_per_us * policy * busy);
   if (t < stream) t = stream;
   if (splits > 1) t += 3.0f + 2.0f * (float)splits * (float)M * (float)N * 4.0f / 5.0e6f;
@@ -2660,7 +2677,14 @@ inline TiledPlan plan_tiled(int64_t M, int64_t N, int64_t K, int force_config, i
       if (force_splits <= 0 && splits != want) continue;  // duplicate of a smaller request
       // (128x256 tiles are the plan for whole rows of K against wide panels; split, they measured behind what
       // their estimate says: 128 x 8192 x 28672 66.3 us against 56.5 with 128x128 tiles)
-      if (c >= 4 && force_splits <= 0 && splits > 1) continue;  // (192x256 tiles were not measured split either)
+      // (192x256 tiles were not measured split either)
+      if ((c == 4 || c == 5) && force_splits <= 0 && splits > 1) continue;
+      // (the deep ring takes three steps to fill: short rows of K stay with the two-step form, 2048 x 2048 x 512
+      // 6.5 us against 6.9)
+      if (c == kDeepSmallConfig && force_config < 0 && sps < 8) continue;
+      // (with one or two tile rows B is fetched with the streaming policy, which this form was not measured
+      // ahead with: 256 x 4096 x 8192 37.7 us against 20.1 for the 64x256 tiles)
+      if (c == kDeepSmallConfig && force_config < 0 && M <= 2 * 128) continue;
       const float cost = plan_cost_us(M, N, K, c, splits, sps);
       if (best_cost < 0.0f || cost < best_cost) {
         best_cost = cost;
@@ -2764,12 +2788,12 @@ int launch_tiled(GemmParams p, hipStream_t stream) {
   return MI355X_FP8_OK;
 }
 
-template <int BM, int BN, int WAVES_M, int WAVES_N, bool STREAM_B>
+template <int BM, int BN, int WAVES_M, int WAVES_N, bool STREAM_B, bool DEEP = false>
 int launch_tiled_epilogue(const GemmParams& p, hipStream_t s) {
   // 256x128 tiles have the LDS for loads three steps ahead (3 A + 4 B stages = 160 KB): worth 6-10 % where
   // the operands come from HBM rather than the memory-side cache (M=1024, N=K=8192 cold: 65.9 -> 60.5 us;
   // K=28672: 220 -> 199 us). The 64x256 tile measured 1-3 % slower that way and stays at two.
-  constexpr int D = (BM == 256 && BN == 128) ? 3 : kDefaultDist;
+  constexpr int D = DEEP || (BM == 256 && BN == 128) ? 3 : kDefaultDist;
   const bool ktail = p.K % kStepK;
   if (p.splits > 1)
     return ktail ? launch_tiled<BM, BN, WAVES_M, WAVES_N, true, kEpiPartial, false, false, D, STREAM_B>(p, s)
@@ -2781,12 +2805,13 @@ int launch_tiled_epilogue(const GemmParams& p, hipStream_t s) {
                : launch_tiled<BM, BN, WAVES_M, WAVES_N, false, kEpiPlain, false, false, D, STREAM_B>(p, s);
 }
 
-template <int BM, int BN, int WAVES_M, int WAVES_N, bool MAY_STREAM>
+template <int BM, int BN, int WAVES_M, int WAVES_N, bool MAY_STREAM, bool DEEP = false>
 int launch_tiled_config(const GemmParams& p, hipStream_t s) {
   if constexpr (MAY_STREAM) {
-    if ((p.M + BM - 1) / BM <= stream_tile_rows(BM, BN)) return launch_tiled_epilogue<BM, BN, WAVES_M, WAVES_N, true>(p, s);
+    if ((p.M + BM - 1) / BM <= stream_tile_rows(BM, BN))
+      return launch_tiled_epilogue<BM, BN, WAVES_M, WAVES_N, true, DEEP>(p, s);
   }
-  return launch_tiled_epilogue<BM, BN, WAVES_M, WAVES_N, false>(p, s);
+  return launch_tiled_epilogue<BM, BN, WAVES_M, WAVES_N, false, DEEP>(p, s);
 }
 
 template <int MT, int NTW, int DEPTH, int KW>
@@ -3092,6 +3117,7 @@ int run_gemm(const void* a, const void* b, const float* a_scale, const float* b_
           case 3: return launch_tiled_config<64, 256, 1, 4, true>(p, s);
           case 4: return launch_tiled_config<128, 256, 2, 2, true>(p, s);
           case 5: return launch_tiled_config<192, 256, 2, 2, true>(p, s);
+          case 6: return launch_tiled_config<128, 128, 2, 2, true, true>(p, s);
           default: return fail(MI355X_FP8_EINVAL, "unknown tile configuration %d", plan.config);
         }
       }
