@@ -2591,6 +2591,9 @@ inline float skinny_streaming_cost_us(int64_t M, int64_t N, int64_t K) {
     const long wgs = (N + (b == 3 ? 31 : 15)) / (b == 3 ? 32 : 16);
     const long rounds = (wgs + kNumCu - 1) / kNumCu;
     if (b >= 2 || rounds > 1) r *= (float)wgs / (float)(rounds * kNumCu);
+    // (long rows on part of the chip: a workgroup streams 23 KB per microsecond at most; 32 x 2304 x 16384 takes
+    // 16.2 us with 144 workgroups, 128x128 tiles in splits 14.7)
+    else if (K > 8192 && wgs < kNumCu) r = fminf(r, (float)wgs * 2.35e4f);
   }
   return 5.0f + (float)N * (float)K / r;
 }
