@@ -295,6 +295,18 @@ def time_quantiser(r, k, dtype, dev, steps=60, copies=3):
     return dict(us=ms * 1e3, gbps=nbytes / ms / 1e6, bound="hbm", frac=nbytes / ms / 1e6 / PEAK_HBM_GBPS)
 
 
+def time_block_quantiser(r, k, dtype, dev, steps=60, copies=3):
+    """128 x 128 block-wise quantiser (the input step of the block-scaled GEMM): algorithmic bytes =
+    source + fp8 output + one f32 scale per block; sources rotate."""
+    from tritonbench_amd import ops
+
+    g = _generator(dev, r, k, 9)
+    xs = [torch.randn((r, k), generator=g, device=dev, dtype=torch.float32).to(dtype) for _ in range(copies)]
+    ms = timed_calls(lambda i: ops.fp8_block_quantize(xs[i % copies]), steps)
+    nbytes = r * k * (xs[0].element_size() + 1) + 4 * (-(-r // 128)) * (-(-k // 128))
+    return dict(us=ms * 1e3, gbps=nbytes / ms / 1e6, bound="hbm", frac=nbytes / ms / 1e6 / PEAK_HBM_GBPS)
+
+
 def time_fused_front_end(which, r, k, dev, steps=60, copies=3):
     """Fused front ends (RMSNorm or SiLU-mul, then the row-wise quantiser, one kernel): algorithmic
     bytes = the bf16 source row(s) + fp8 output + one f32 scale per row (the RMSNorm weight vector is
@@ -656,6 +668,8 @@ def main():
         attempt("quantise_f32_8192x8192", lambda: time_quantiser(8192, 8192, torch.float32, dev))
         attempt("quantise_bf16_8192x8192", lambda: time_quantiser(8192, 8192, torch.bfloat16, dev))
         attempt("quantise_bf16_57344x8192", lambda: time_quantiser(57344, 8192, torch.bfloat16, dev, steps=20, copies=2))
+        attempt("block_quantise_bf16_8192x8192", lambda: time_block_quantiser(8192, 8192, torch.bfloat16, dev))
+        attempt("block_quantise_f32_8192x8192", lambda: time_block_quantiser(8192, 8192, torch.float32, dev))
         attempt("rmsnorm_quantise_bf16_8192x8192", lambda: time_fused_front_end("rmsnorm", 8192, 8192, dev))
         attempt("silu_mul_quantise_bf16_8192x8192", lambda: time_fused_front_end("silu_mul", 8192, 8192, dev))
         # (rows of 2048 elements: the forms with a wave per row; eight sources in rotation, 0.5 GB)

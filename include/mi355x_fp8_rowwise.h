@@ -256,6 +256,31 @@ int mi355x_fp8_blockwise_gemm(const void* a, const void* b,
                               int64_t lda, int64_t ldb, int64_t ldc, void* stream);
 
 /*
+ * Block-wise e4m3fn quantiser, replacing fp8_block_quantize
+ * (tritonbench/operators/fp8_gemm_blockwise/operator.py:86-118): one scale per 128 x 128 block,
+ *
+ *   amax[i,j]      = max |x| over block (i, j); elements past M or K count as zero
+ *   scale[i,j]     = fl(fl(1 / max(amax[i,j], 1e-12)) * 448), +inf replaced by 1     (f32)
+ *   xq[m,k]        = e4m3fn( x[m,k] * scale[m/128][k/128] )      (f32 product, round to nearest even)
+ *   inv_scale[i,j] = 1 / scale[i,j]                                (f32)
+ *
+ * The lower bound 1e-12 is taken in the source type (for a bf16 source it is the bf16 nearest to
+ * 1e-12), everything after it in f32, as eager PyTorch evaluates that function. A block holding a
+ * NaN comes out as NaN codes with a NaN inverse scale; a block holding an infinity gets scale 0
+ * and inverse scale +inf, its finite elements become zero and the infinities NaN.
+ *
+ *   x          [M, K] of `src_type`, row stride ldx (elements)     xq  e4m3fn [M, K], row stride ldq
+ *   inv_scale  f32 [ceil(M/128)][ceil(K/128)], contiguous: what mi355x_fp8_blockwise_gemm takes
+ *
+ * At most 65535 block rows (M <= 8388480). Rows 16-byte aligned with K a whole number of 16-byte
+ * source chunks take the one-pass form; anything else a slower element-wise one.
+ */
+int mi355x_fp8_blockwise_quantize(const void* x, int src_type,
+                                  void* xq, float* inv_scale,
+                                  int64_t M, int64_t K, int64_t ldx, int64_t ldq,
+                                  void* stream);
+
+/*
  * Row-wise e4m3fn quantiser, replacing fp8_row_quantize (operator.py:136-145):
  *   amax[r]      = max_k |x[r,k]|
  *   scale[r]     = fl(fl(1 / max(amax[r], 1e-12)) * 448)   (how PyTorch evaluates 448 / tensor)

@@ -96,6 +96,10 @@ SIGNATURES = {
         [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
          c_int64, c_int64, c_int64, c_int64, c_int64, c_int64, c_void_p],
     ),
+    "mi355x_fp8_blockwise_quantize": (
+        c_int,
+        [c_void_p, c_int, c_void_p, c_void_p, c_int64, c_int64, c_int64, c_int64, c_void_p],
+    ),
     "mi355x_fp8_rowwise_quantize": (
         c_int,
         [c_void_p, c_int, c_void_p, c_void_p, c_int64, c_int64, c_int64, c_int64, c_void_p],

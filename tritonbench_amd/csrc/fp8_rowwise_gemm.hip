@@ -2265,6 +2265,117 @@ __global__ __launch_bounds__(THREADS* ROWS) void quantize_rows_vec_kernel(const 
 
 
 // ------------------------------------------------------------------------------------
+// Block-wise quantiser: one scale per 128 x 128 block of the source, the input step of the
+// block-scaled GEMM. One workgroup per block keeps the block in registers between the
+// maximum and the conversion, so the source is read once. Follows the eager PyTorch program of
+// tritonbench/operators/fp8_gemm_blockwise/operator.py:86-118:
+//   amax  = max |x| over the block (elements past M or K count as zero), clamped from below
+//           with 1e-12 in the source type, then widened to f32
+//   scale = fl(fl(1 / amax) * 448) in f32 (how PyTorch evaluates 448 / tensor); +inf -> 1
+//   xq    = e4m3fn(fl(x * scale)), the product in f32 whatever the source type, no clamp
+//           (|x * scale| cannot reach 464, the first value the cast turns into NaN)
+//   inv   = fl(1 / scale)
+// A block that holds a NaN comes out as NaN codes with a NaN inverse scale; a block that holds an
+// infinity gets scale 0 and inverse scale +inf, its finite elements become zero, the infinities NaN.
+// ------------------------------------------------------------------------------------
+constexpr int kQuantBlock = 128;
+
+template <typename SrcT>
+__device__ __forceinline__ float block_scale(float amax) {
+  const float floor_ = SrcTraits<SrcT>::round(1e-12f);
+  const float clamped = amax < floor_ ? floor_ : amax;  // false for NaN: it stays
+  const float scale = (1.0f / clamped) * 448.0f;
+  return scale == __builtin_inff() ? 1.0f : scale;
+}
+
+// VEC: 16-byte source chunks (rows 16-byte aligned, K a whole number of chunks), 4- or 8-byte stores.
+// Otherwise element by element, the block read twice (the second time from cache).
+template <typename SrcT, bool VEC>
+__global__ __launch_bounds__(256) void quantize_blocks_kernel(const SrcT* x, uint8_t* xq, float* inv_scale, int M,
+                                                              int K, long ldx, long ldq, int grid_k) {
+  using T = SrcTraits<SrcT>;
+  using V = VecTraits<SrcT>;
+  constexpr int EPV = V::EPV;
+  constexpr int CPR = kQuantBlock / EPV;   // chunks per block row
+  constexpr int RPP = 256 / CPR;           // block rows per pass of the workgroup
+  constexpr int PASSES = kQuantBlock / RPP;
+  __shared__ float wave_max[4];
+  const int bk = blockIdx.x, bm = blockIdx.y;
+  const int m0 = bm * kQuantBlock, k0 = bk * kQuantBlock;
+  const int tid = threadIdx.x;
+  const int chunk = tid % CPR, row0 = tid / CPR;
+
+  v4i cache[VEC ? PASSES : 1];
+  float amax = 0.0f;
+  if constexpr (VEC) {
+#pragma unroll
+    for (int i = 0; i < PASSES; ++i) {
+      const int r = m0 + row0 + i * RPP, c = k0 + chunk * EPV;
+      const bool inside = r < M && c < K;
+      // (outside the matrix a lane reads the block's first chunk, which exists, and drops it)
+      const v4i got = __builtin_nontemporal_load((const v4i*)(x + (inside ? (long)r * ldx + c : (long)m0 * ldx + k0)));
+      cache[i] = inside ? got : (v4i){0, 0, 0, 0};
+      float f[EPV];
+      V::unpack(cache[i], f);
+#pragma unroll
+      for (int e = 0; e < EPV; ++e) amax = max_keep_nan(amax, fabsf(f[e]));
+    }
+  } else {
+    for (int idx = tid; idx < kQuantBlock * kQuantBlock; idx += 256) {
+      const int r = m0 + idx / kQuantBlock, c = k0 + idx % kQuantBlock;
+      if (r < M && c < K) amax = max_keep_nan(amax, fabsf(T::load(x + (long)r * ldx + c)));
+    }
+  }
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) amax = max_keep_nan(amax, __shfl_xor(amax, o));
+  if ((tid & 63) == 0) wave_max[tid >> 6] = amax;
+  __syncthreads();
+  amax = max_keep_nan(max_keep_nan(wave_max[0], wave_max[1]), max_keep_nan(wave_max[2], wave_max[3]));
+
+  const float scale = block_scale<SrcT>(amax);
+  if (tid == 0) inv_scale[(long)bm * grid_k + bk] = 1.0f / scale;
+  const bool finite = amax < __builtin_inff();  // false for NaN and infinity: the integer encoder carries them
+
+  if constexpr (VEC) {
+#pragma unroll
+    for (int i = 0; i < PASSES; ++i) {
+      const int r = m0 + row0 + i * RPP, c = k0 + chunk * EPV;
+      if (r >= M || c >= K) continue;
+      float f[EPV];
+      V::unpack(cache[i], f);
+      uint32_t out[EPV / 4];
+      if (finite) {
+#pragma unroll
+        for (int w = 0; w < EPV / 4; ++w) {
+          // (the clamp changes nothing for a finite block; it keeps the pack-convert inside its range)
+          float g[4];
+#pragma unroll
+          for (int e = 0; e < 4; ++e) g[e] = fminf(fmaxf(f[4 * w + e] * scale, -448.0f), 448.0f);
+          int packed = __builtin_amdgcn_cvt_pk_fp8_f32(g[0], g[1], 0, false);
+          packed = __builtin_amdgcn_cvt_pk_fp8_f32(g[2], g[3], packed, true);
+          out[w] = (uint32_t)packed;
+        }
+      } else {
+#pragma unroll
+        for (int w = 0; w < EPV / 4; ++w) {
+          out[w] = 0;
+#pragma unroll
+          for (int e = 0; e < 4; ++e) out[w] |= (uint32_t)f32_to_e4m3fn_rne(f[4 * w + e] * scale) << (8 * e);
+        }
+      }
+      uint8_t* dst = xq + (long)r * ldq + c;
+      if (EPV == 4) *(uint32_t*)dst = out[0];
+      else *(v2u*)dst = (v2u){out[0], out[EPV / 4 - 1]};
+    }
+  } else {
+    for (int idx = tid; idx < kQuantBlock * kQuantBlock; idx += 256) {
+      const int r = m0 + idx / kQuantBlock, c = k0 + idx % kQuantBlock;
+      if (r < M && c < K) xq[(long)r * ldq + c] = f32_to_e4m3fn_rne(T::load(x + (long)r * ldx + c) * scale);
+    }
+  }
+}
+
+// ------------------------------------------------------------------------------------
 // Fused front ends of the row-wise GEMM: the activation is normalised (RMSNorm with a weight
 // vector) or gated (SiLU(x1) * x2) and quantised row-wise in one pass, so the bf16 row is read
 // from memory once and nothing but the e4m3fn codes and one scale per row is written.
@@ -3338,6 +3449,36 @@ int mi355x_fp8_rowwise_quantize(const void* x, int src_type, void* xq, float* in
   }
   hipError_t e = hipGetLastError();
   if (e != hipSuccess) return fail(MI355X_FP8_ELAUNCH, "quantize kernel launch: %s", hipGetErrorString(e));
+  return MI355X_FP8_OK;
+}
+
+int mi355x_fp8_blockwise_quantize(const void* x, int src_type, void* xq, float* inv_scale, int64_t M, int64_t K,
+                                  int64_t ldx, int64_t ldq, void* stream) {
+  if (!x || !xq || !inv_scale) return fail(MI355X_FP8_EINVAL, "null pointer");
+  if (M < 1 || K < 1 || ldx < K || ldq < K) return fail(MI355X_FP8_EINVAL, "bad shape or leading dimension");
+  if (M > INT32_MAX || K > INT32_MAX) return fail(MI355X_FP8_ENOTSUP, "dimension exceeds 2^31-1");
+  if (src_type != MI355X_FP8_SRC_F32 && src_type != MI355X_FP8_SRC_BF16)
+    return fail(MI355X_FP8_EINVAL, "unknown src_type %d", src_type);
+  const int64_t grid_m = (M + kQuantBlock - 1) / kQuantBlock, grid_k = (K + kQuantBlock - 1) / kQuantBlock;
+  if (grid_m > 65535) return fail(MI355X_FP8_ENOTSUP, "more than 65535 block rows");
+  hipStream_t s = (hipStream_t)stream;
+  const int esz = src_type == MI355X_FP8_SRC_BF16 ? 2 : 4;
+  const int epv = 16 / esz;
+  // whole 16-byte source chunks from 16-byte aligned rows, and stores of a chunk's codes (4 or 8 bytes) aligned
+  const bool vec = (reinterpret_cast<uintptr_t>(x) & 15) == 0 && (ldx * esz) % 16 == 0 && K % epv == 0 &&
+                   (reinterpret_cast<uintptr_t>(xq) & (epv - 1)) == 0 && ldq % epv == 0;
+  const dim3 grid((unsigned)grid_k, (unsigned)grid_m);
+  if (src_type == MI355X_FP8_SRC_F32) {
+    auto kern = vec ? quantize_blocks_kernel<float, true> : quantize_blocks_kernel<float, false>;
+    hipLaunchKernelGGL(kern, grid, dim3(256), 0, s, (const float*)x, (uint8_t*)xq, inv_scale, (int)M, (int)K, (long)ldx,
+                       (long)ldq, (int)grid_k);
+  } else {
+    auto kern = vec ? quantize_blocks_kernel<uint16_t, true> : quantize_blocks_kernel<uint16_t, false>;
+    hipLaunchKernelGGL(kern, grid, dim3(256), 0, s, (const uint16_t*)x, (uint8_t*)xq, inv_scale, (int)M, (int)K,
+                       (long)ldx, (long)ldq, (int)grid_k);
+  }
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess) return fail(MI355X_FP8_ELAUNCH, "block quantize kernel launch: %s", hipGetErrorString(e));
   return MI355X_FP8_OK;
 }
 

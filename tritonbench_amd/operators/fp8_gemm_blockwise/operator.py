@@ -44,9 +44,9 @@ def parse_args(args: List[str]) -> argparse.Namespace:
     return p.parse_args(args)
 
 
-def fp8_block_quantize(x: torch.Tensor, block_m: int = BLOCK, block_k: int = BLOCK) -> Tuple[torch.Tensor, torch.Tensor]:
-    """One scale per block_m x block_k block, on whatever device x lives on; returns the fp8
-    tensor and the inverse scales [ceil(M/block_m), ceil(K/block_k)] (operator.py:86-118)."""
+def fp8_block_quantize_torch(x: torch.Tensor, block_m: int = BLOCK, block_k: int = BLOCK) -> Tuple[torch.Tensor, torch.Tensor]:
+    """Eager PyTorch form (operator.py:86-118): one scale per block_m x block_k block; returns the
+    fp8 tensor and the inverse scales [ceil(M/block_m), ceil(K/block_k)]. Used for host tensors."""
     m, k = x.shape
     gm, gk = -(-m // block_m), -(-k // block_k)
     padded = torch.zeros(gm * block_m, gk * block_k, dtype=x.dtype, device=x.device)
@@ -56,6 +56,13 @@ def fp8_block_quantize(x: torch.Tensor, block_m: int = BLOCK, block_k: int = BLO
     scale[scale == float("inf")] = 1.0
     xq = (padded * scale.repeat_interleave(block_m, dim=0).repeat_interleave(block_k, dim=1))[:m, :k]
     return xq.to(torch.float8_e4m3fn), 1 / scale
+
+
+def fp8_block_quantize(x: torch.Tensor) -> Tuple[torch.Tensor, torch.Tensor]:
+    """128 x 128 block quantisation: the HIP kernel for device tensors, eager PyTorch for host tensors."""
+    if x.is_cuda:
+        return ops.fp8_block_quantize(x)
+    return fp8_block_quantize_torch(x)
 
 
 class Operator(BenchmarkOperator):

@@ -302,6 +302,31 @@ def fp8_row_quantize(x: torch.Tensor) -> Tuple[torch.Tensor, torch.Tensor]:
     return xq, inv_scale
 
 
+def fp8_block_quantize(x: torch.Tensor) -> Tuple[torch.Tensor, torch.Tensor]:
+    """128 x 128 block-wise e4m3fn quantisation on the GPU; returns (xq, inverse scales
+    [ceil(M/128), ceil(K/128)]) like fp8_block_quantize in
+    tritonbench/operators/fp8_gemm_blockwise/operator.py:86-118."""
+    lib = _lib.load()
+    _require_gpu(x, "x")
+    if x.dim() != 2 or x.stride(1) != 1:
+        raise ValueError("x must be 2-D with unit column stride")
+    if x.dtype == torch.float32:
+        src = _lib.SRC_F32
+    elif x.dtype == torch.bfloat16:
+        src = _lib.SRC_BF16
+    else:
+        raise TypeError(f"unsupported source dtype {x.dtype}")
+    m, k = x.shape
+    xq = torch.empty((m, k), dtype=FP8_DTYPE, device=x.device)
+    inv_scale = torch.empty((-(-m // BLOCK), -(-k // BLOCK)), dtype=torch.float32, device=x.device)
+    st = lib.mi355x_fp8_blockwise_quantize(
+        x.data_ptr(), src, xq.data_ptr(), inv_scale.data_ptr(), m, k, x.stride(0), xq.stride(0),
+        _stream_ptr(),
+    )
+    _lib.check(st, "mi355x_fp8_blockwise_quantize")
+    return xq, inv_scale
+
+
 def _fused_quant_outputs(x: torch.Tensor) -> Tuple[torch.Tensor, torch.Tensor]:
     r, k = x.shape
     return (torch.empty((r, k), dtype=FP8_DTYPE, device=x.device),
