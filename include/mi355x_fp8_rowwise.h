@@ -53,6 +53,9 @@ extern "C" {
 #define MI355X_FP8_VARIANT_TILED   1  /* LDS-tiled persistent MFMA kernel (compute-bound shapes) */
 #define MI355X_FP8_VARIANT_SKINNY  2  /* kernels that own all of K per workgroup and stream B (HBM-bound): M <= 64, \
                                          and M <= 256 where the narrow-tile form below fits */
+#define MI355X_FP8_VARIANT_GENERIC 3  /* byte loads and f32 multiply-adds, no requirement on K, the leading dimensions or \
+                                         the alignment of a and b: what AUTO runs for operands the two MFMA families   \
+                                         cannot take (a few TFLOP/s) */
 
 /*
  * The `variant` argument is a word: bits 0..7 hold the family above; for the tiled family
@@ -111,8 +114,9 @@ int mi355x_fp8_rowwise_init(void);
 
 const char* mi355x_fp8_rowwise_last_error(void);
 
-/* Variant AUTO would run for this shape (one of the MI355X_FP8_VARIANT_* values > 0),
- * or a negative status when the shape is not supported. Lets tests pin the dispatch. */
+/* Variant AUTO would run for this shape with operands that meet the MFMA families' alignment
+ * requirements (one of the MI355X_FP8_VARIANT_* values > 0; GENERIC when K is not a multiple
+ * of 16), or a negative status when the shape is not supported. Lets tests pin the dispatch. */
 int mi355x_fp8_rowwise_select_variant(int64_t M, int64_t N, int64_t K);
 
 /* Bytes of device workspace `variant` needs for this shape (0 when none). Pure host
@@ -129,7 +133,10 @@ size_t mi355x_fp8_rowwise_workspace_bytes(int64_t M, int64_t N, int64_t K, int v
  *   a_scale  f32 [M]                            b_scale  f32 [N]
  *   bias     bf16 [N] or NULL                   c        bf16 [M, N], row stride ldc
  *
- * Requirements: M, N, K >= 1; K, lda, ldb multiples of 16; a and b 16-byte aligned.
+ * Requirements: M, N, K >= 1. The MFMA families (TILED, SKINNY) want K, lda, ldb multiples of
+ * 16, a and b 16-byte aligned and lda*256, ldb*256, ldc*512 below 2^31; pinned, they answer
+ * ENOTSUP otherwise. AUTO sends operands that miss any of that to the GENERIC family, which
+ * takes every K, leading dimension and alignment (M <= 4194240).
  * `workspace` (16-byte aligned) may be NULL when mi355x_fp8_rowwise_workspace_bytes() is 0.
  * A call whose variant leaves the split-K factor to the library and brings less workspace
  * than that runs the best plan that needs none (same results up to fp32 summation order);
@@ -248,7 +255,7 @@ int mi355x_fp8_rowwise_grouped_gemm(const void* a, const void* b,
  *   a_scale  f32 [ceil(M/128)][ceil(K/128)]       b_scale  f32 [ceil(N/128)][ceil(K/128)]
  *   c        bf16 [M, N]
  *
- * Requirements as for mi355x_fp8_rowwise_gemm, and K <= 32768.
+ * Requirements as for the MFMA families of mi355x_fp8_rowwise_gemm, and K <= 32768.
  */
 int mi355x_fp8_blockwise_gemm(const void* a, const void* b,
                               const float* a_scale, const float* b_scale, void* c,

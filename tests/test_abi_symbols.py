@@ -34,6 +34,7 @@ def test_abi_version_and_status_constants_match_header():
     assert int(consts["MI355X_FP8_ELAUNCH"]) == _lib.ELAUNCH
     assert int(consts["MI355X_FP8_VARIANT_TILED"]) == _lib.VARIANT_TILED
     assert int(consts["MI355X_FP8_VARIANT_SKINNY"]) == _lib.VARIANT_SKINNY
+    assert int(consts["MI355X_FP8_VARIANT_GENERIC"]) == _lib.VARIANT_GENERIC
     assert int(consts["MI355X_FP8_SRC_BF16"]) == _lib.SRC_BF16
 
 
@@ -55,12 +56,14 @@ def test_host_side_argument_checks_need_no_gpu():
             assert lib.mi355x_fp8_rowwise_select_variant(m, n, 1024) == _lib.VARIANT_TILED
     assert lib.mi355x_fp8_rowwise_select_variant(64, 57344, 8192) == _lib.VARIANT_TILED
     assert lib.mi355x_fp8_rowwise_select_variant(0, 8, 16) == _lib.EINVAL
-    assert lib.mi355x_fp8_rowwise_select_variant(8, 8, 24) == _lib.ENOTSUP
-    assert "multiple of 16" in _lib.last_error()
+    assert lib.mi355x_fp8_rowwise_select_variant(8, 8, 24) == _lib.VARIANT_GENERIC  # K not a multiple of 16
+    assert lib.mi355x_fp8_rowwise_workspace_bytes(128, 8192, 8200, _lib.VARIANT_AUTO) == 0
+    assert lib.mi355x_fp8_rowwise_select_variant(2 ** 31, 8, 16) == _lib.ENOTSUP
+    assert "2^31" in _lib.last_error()
     st = lib.mi355x_fp8_rowwise_gemm(None, None, None, None, None, None, 16, 16, 16, 16, 16, 16, None, 0, 0, None)
     assert st == _lib.EINVAL and "null" in _lib.last_error()
     st = lib.mi355x_fp8_rowwise_gemm(None, None, None, None, None, None, 16, 16, 20, 32, 32, 16, None, 0, 0, None)
-    assert st == _lib.ENOTSUP
+    assert st == _lib.EINVAL  # (null pointers; K = 20 alone is the generic family's business)
 
 
 def test_status_to_exception_mapping():
@@ -68,7 +71,7 @@ def test_status_to_exception_mapping():
 
     lib = _lib.load()
     with pytest.raises(NotImplementedError):
-        _lib.check(lib.mi355x_fp8_rowwise_select_variant(8, 8, 24), "select")
+        _lib.check(lib.mi355x_fp8_rowwise_select_variant(8, 2 ** 31, 16), "select")
     with pytest.raises(ValueError):
         _lib.check(lib.mi355x_fp8_rowwise_select_variant(-1, 8, 16), "select")
     _lib.check(0, "fine")
@@ -115,8 +118,9 @@ def test_grouped_and_blockwise_argument_checks_need_no_gpu():
 
 def test_leading_dimension_limits_are_checked_on_the_host():
     """A tile's rows are addressed with 32-bit byte offsets: 256 rows of A or B and 256 rows of
-    16-bit output must stay below 2^31 bytes. The check comes before any device call, so host
-    buffers (never dereferenced) can stand in for the operands."""
+    16-bit output must stay below 2^31 bytes for the MFMA families (pinned here: the automatic
+    choice would hand such operands to the generic family). The check comes before any device
+    call, so host buffers (never dereferenced) can stand in for the operands."""
     lib = _lib.load()
     buf = ctypes.create_string_buffer(4096 + 64)
     base = (ctypes.addressof(buf) + 63) & ~63  # 64-byte aligned stand-in for every operand
@@ -125,7 +129,8 @@ def test_leading_dimension_limits_are_checked_on_the_host():
     limit_c = (2 ** 31 - 1) // 512
 
     def call(lda, ldb, ldc):
-        return lib.mi355x_fp8_rowwise_gemm(base, base, base, base, None, base, m, n, k, lda, ldb, ldc, None, 0, 0, None)
+        return lib.mi355x_fp8_rowwise_gemm(base, base, base, base, None, base, m, n, k, lda, ldb, ldc, None, 0,
+                                           _lib.VARIANT_TILED, None)
 
     too_wide = (limit_ab // 16 + 1) * 16
     assert call(too_wide, 16, 16) == _lib.ENOTSUP and "leading dimension too large" in _lib.last_error()

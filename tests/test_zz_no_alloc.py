@@ -148,5 +148,5 @@ def test_no_alloc_entry_refuses_plans_beyond_its_buffer():
     msg = _lib.last_error()
     assert str(need) in msg and str(_lib.NOALLOC_SCRATCH_BYTES) in msg
     # bad shapes and variants keep their usual status
-    assert lib.mi355x_fp8_rowwise_gemm_noalloc(None, None, None, None, None, None, 16, 16, 24, 32, 32, 16, 0, None) == _lib.ENOTSUP
+    assert lib.mi355x_fp8_rowwise_gemm_noalloc(None, None, None, None, None, None, 16, 2 ** 31, 32, 32, 32, 16, 0, None) == _lib.ENOTSUP
     assert lib.mi355x_fp8_rowwise_gemm_noalloc(None, None, None, None, None, None, 16, 16, 16, 16, 16, 16, 1 << 25, None) == _lib.EINVAL

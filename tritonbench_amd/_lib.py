@@ -21,6 +21,7 @@ ELAUNCH = -3
 VARIANT_AUTO = 0
 VARIANT_TILED = 1
 VARIANT_SKINNY = 2
+VARIANT_GENERIC = 3  # byte loads + f32 multiply-adds: any K, leading dimension and alignment
 SKINNY_ONE_TILE = 1 << 8  # skinny family: pins the one-tile-per-workgroup kernel
 SKINNY_NARROW = 2 << 8  # skinny family: pins the narrow-tile kernel (the shapes `skinny_family_takes`)
 SKINNY_RESIDENT = 4 << 8  # skinny family: pins the forms that keep A on chip (pair / persistent kernel)

@@ -1142,6 +1142,71 @@ __global__ __launch_bounds__(256) void splitk_finalize_kernel(GemmParams p) {
 }
 
 // ------------------------------------------------------------------------------------
+// Generic kernel: operands the other families cannot take (K, lda or ldb not a multiple of 16,
+// A or B not 16-byte aligned, leading dimensions beyond a buffer descriptor's range). Byte loads,
+// codes widened to f32 in LDS, f32 multiply-adds (the product of two e4m3fn values is exact in
+// f32), 64x64 tile per workgroup, 4x4 outputs per lane. A few TFLOP/s: a correct answer for
+// odd shapes, not a fast one. Same epilogue arithmetic as the other kernels.
+// ------------------------------------------------------------------------------------
+__device__ __forceinline__ float e4m3fn_to_f32(uint8_t code) {
+  const uint32_t mag = code & 0x7fu;
+  // the 7 magnitude bits placed at an f32's exponent/mantissa boundary are the value times 2^-120
+  // (subnormal codes become subnormal floats, which the multiply takes as they are)
+  float v = __uint_as_float(mag << 20) * 0x1p120f;
+  if (mag == 0x7fu) v = __uint_as_float(0x7fc00000u);
+  return (code & 0x80u) ? -v : v;
+}
+
+constexpr int kGenericTile = 64, kGenericStepK = 32;
+
+__global__ __launch_bounds__(256) void gemm_generic_kernel(GemmParams p) {
+  __shared__ float as[kGenericStepK][kGenericTile + 1];
+  __shared__ float bs[kGenericStepK][kGenericTile + 1];
+  const int tid = threadIdx.x;
+  const long m0 = (long)blockIdx.y * kGenericTile, n0 = (long)blockIdx.x * kGenericTile;
+  const int ld_row = tid / 4, ld_k = (tid % 4) * 8;  // the 8 bytes of one tile row a lane widens per step
+  const int ty = tid / 16, tx = tid % 16;
+  float acc[4][4] = {};
+  for (long k0 = 0; k0 < p.K; k0 += kGenericStepK) {
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      const long k = k0 + ld_k + e;
+      const bool in_k = k < p.K;
+      as[ld_k + e][ld_row] = in_k && m0 + ld_row < p.M ? e4m3fn_to_f32(p.a[(size_t)(m0 + ld_row) * p.lda + k]) : 0.0f;
+      bs[ld_k + e][ld_row] = in_k && n0 + ld_row < p.N ? e4m3fn_to_f32(p.b[(size_t)(n0 + ld_row) * p.ldb + k]) : 0.0f;
+    }
+    __syncthreads();
+#pragma unroll 8
+    for (int kk = 0; kk < kGenericStepK; ++kk) {
+      float av[4], bv[4];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) av[i] = as[kk][ty * 4 + i];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) bv[j] = bs[kk][tx * 4 + j];
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) acc[i][j] = __builtin_fmaf(av[i], bv[j], acc[i][j]);
+    }
+    __syncthreads();
+  }
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const long m = m0 + ty * 4 + i;
+    if (m >= p.M) continue;
+    const float sa_m = p.a_scale[m];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const long n = n0 + tx * 4 + j;
+      if (n >= p.N) continue;
+      const float t = acc[i][j] * sa_m;
+      const float r = p.bias ? __builtin_fmaf(t, p.b_scale[n], bf16_to_f32(p.bias[n])) : t * p.b_scale[n];
+      p.c[(size_t)m * p.ldc + n] = (uint16_t)pack_out_x2(r, 0.0f, p.out_f16);
+    }
+  }
+}
+
+// ------------------------------------------------------------------------------------
 // Skinny kernel (M <= 16*MT, HBM-bound): B is streamed exactly once and nothing is reused, so
 // what matters is whole-line coalesced loads and as many bytes in flight as a plain copy has.
 //
@@ -2564,6 +2629,10 @@ int check_shape(int64_t M, int64_t N, int64_t K) {
                                            (long long)M, (long long)N, (long long)K);
   if (M > INT32_MAX || N > INT32_MAX || K > INT32_MAX)
     return fail(MI355X_FP8_ENOTSUP, "dimension exceeds 2^31-1");
+  return MI355X_FP8_OK;
+}
+// What the MFMA families ask of the operands beyond check_shape (the generic family asks nothing).
+int check_fast_shape(int64_t K) {
   if (K % 16 != 0) return fail(MI355X_FP8_ENOTSUP, "K must be a multiple of 16 (got %lld)", (long long)K);
   return MI355X_FP8_OK;
 }
@@ -3101,6 +3170,7 @@ const char* mi355x_fp8_rowwise_last_error(void) { return g_err; }
 int mi355x_fp8_rowwise_select_variant(int64_t M, int64_t N, int64_t K) {
   const int st = check_shape(M, N, K);
   if (st != MI355X_FP8_OK) return st;
+  if (K % 16 != 0) return MI355X_FP8_VARIANT_GENERIC;
   // M <= 64: the streaming kernel, unless a tiled plan (64- or 128-row tiles that stream B, split
   // K where the tiles are few) is expected to beat it: from two 16-row blocks of A up on most
   // shapes, with one block on the longest weight panels. Up to 8 rows the streaming kernel was
@@ -3116,7 +3186,8 @@ size_t mi355x_fp8_rowwise_workspace_bytes(int64_t M, int64_t N, int64_t K, int v
   if (check_shape(M, N, K) != MI355X_FP8_OK) return 0;
   if ((variant & 0xff) == MI355X_FP8_VARIANT_AUTO)
     variant = (variant & ~0xff) | mi355x_fp8_rowwise_select_variant(M, N, K);
-  if ((variant & 0xff) != MI355X_FP8_VARIANT_TILED) return 0;  // the skinny kernel reduces on chip
+  // (the skinny kernels reduce on chip, the generic kernel does not split)
+  if ((variant & 0xff) != MI355X_FP8_VARIANT_TILED || K % 16 != 0) return 0;
   const TiledPlan plan = plan_from_variant(M, N, K, variant, kMaxSplits);
   return plan.splits > 1 ? (size_t)plan.splits * (size_t)M * (size_t)N * sizeof(float) : 0;
 }
@@ -3160,19 +3231,28 @@ int run_gemm(const void* a, const void* b, const float* a_scale, const float* b_
   if (st != MI355X_FP8_OK) return st;
   if (!a || !b || !a_scale || !b_scale || !c) return fail(MI355X_FP8_EINVAL, "null operand pointer");
   if (lda < K || ldb < K || ldc < N) return fail(MI355X_FP8_EINVAL, "leading dimension smaller than the row length");
-  if (lda % 16 || ldb % 16) return fail(MI355X_FP8_ENOTSUP, "lda and ldb must be multiples of 16");
-  if ((reinterpret_cast<uintptr_t>(a) & 15) || (reinterpret_cast<uintptr_t>(b) & 15))
-    return fail(MI355X_FP8_ENOTSUP, "a and b must be 16-byte aligned");
   if ((reinterpret_cast<uintptr_t>(a_scale) & 3) || (reinterpret_cast<uintptr_t>(b_scale) & 3) ||
       (reinterpret_cast<uintptr_t>(c) & 1) || (reinterpret_cast<uintptr_t>(bias) & 1))
     return fail(MI355X_FP8_EINVAL, "misaligned scale, bias or output pointer");
-  // (a tile's rows are addressed with 32-bit byte offsets that must stay below 2^31)
-  if (lda * 256 > (int64_t)INT32_MAX || ldb * 256 > (int64_t)INT32_MAX || ldc * 512 > (int64_t)INT32_MAX)
-    return fail(MI355X_FP8_ENOTSUP, "leading dimension too large");
   if (variant < 0 || (variant >> 24) || ((variant >> 8) & 0xff) > kNumTileConfigs)
     return fail(MI355X_FP8_EINVAL, "unknown variant 0x%x", variant);
   const int plan_bits = variant & ~0xff;
   variant &= 0xff;
+  // What the MFMA families ask of the operands; the generic family takes whatever is left, and AUTO
+  // sends it there.
+  const char* unfit = nullptr;
+  if (K % 16 != 0) unfit = "K must be a multiple of 16";
+  else if (lda % 16 || ldb % 16) unfit = "lda and ldb must be multiples of 16";
+  else if ((reinterpret_cast<uintptr_t>(a) & 15) || (reinterpret_cast<uintptr_t>(b) & 15)) unfit = "a and b must be 16-byte aligned";
+  // (a tile's rows are addressed with 32-bit byte offsets that must stay below 2^31)
+  else if (lda * 256 > (int64_t)INT32_MAX || ldb * 256 > (int64_t)INT32_MAX || ldc * 512 > (int64_t)INT32_MAX)
+    unfit = "leading dimension too large";
+  if (unfit && variant == MI355X_FP8_VARIANT_AUTO) variant = MI355X_FP8_VARIANT_GENERIC;
+  if (unfit && variant != MI355X_FP8_VARIANT_GENERIC)
+    return fail(MI355X_FP8_ENOTSUP, "%s for this kernel family (lda %lld, ldb %lld, ldc %lld, K %lld); the generic family or "
+                "the automatic choice takes such operands", unfit, (long long)lda, (long long)ldb, (long long)ldc, (long long)K);
+  if (variant == MI355X_FP8_VARIANT_GENERIC && stamps)
+    return fail(MI355X_FP8_ENOTSUP, "the stamped entry point runs the tiled family only");
   if (variant == MI355X_FP8_VARIANT_AUTO) {
     variant = mi355x_fp8_rowwise_select_variant(M, N, K);
     if (variant == MI355X_FP8_VARIANT_TILED && (M <= kSkinnyMaxM || narrow_fits(M, N, K))) {
@@ -3269,6 +3349,15 @@ int run_gemm(const void* a, const void* b, const float* a_scale, const float* b_
       if (M <= 32) return launch_skinny<2, 1, 2, 8>(p, s);
       if (M <= 48) return launch_skinny<3, 1, 2, 8>(p, s);
       return launch_skinny<4, 2, 2, 8>(p, s);  // 32 rows of B per workgroup: A passes L1 half as often
+    case MI355X_FP8_VARIANT_GENERIC: {
+      if (const int gs = ready_device()) return gs;
+      const dim3 grid((unsigned)((N + kGenericTile - 1) / kGenericTile), (unsigned)((M + kGenericTile - 1) / kGenericTile));
+      if (grid.y > 65535) return fail(MI355X_FP8_ENOTSUP, "the generic family takes M <= %d", 65535 * kGenericTile);
+      hipLaunchKernelGGL(gemm_generic_kernel, grid, dim3(256), 0, s, p);
+      const hipError_t e = hipGetLastError();
+      if (e != hipSuccess) return fail(MI355X_FP8_ELAUNCH, "generic kernel launch: %s", hipGetErrorString(e));
+      return MI355X_FP8_OK;
+    }
     default:
       return fail(MI355X_FP8_EINVAL, "unknown variant %d", variant);
   }
@@ -3309,6 +3398,7 @@ int mi355x_fp8_rowwise_grouped_gemm(const void* a, const void* b, const float* a
                                     int64_t K, int64_t lda, int64_t ldb, int64_t ldc, int tile_config,
                                     void* stream) {
   int st = check_shape(M, N, K);
+  if (st == MI355X_FP8_OK) st = check_fast_shape(K);
   if (st != MI355X_FP8_OK) return st;
   if (G < 1 || G > 65536) return fail(MI355X_FP8_EINVAL, "G must be in 1..65536 (got %lld)", (long long)G);
   if (G * N > INT32_MAX) return fail(MI355X_FP8_ENOTSUP, "G*N exceeds 2^31-1");
@@ -3356,6 +3446,7 @@ int mi355x_fp8_blockwise_gemm(const void* a, const void* b, const float* a_scale
                               void* c, int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldb,
                               int64_t ldc, void* stream) {
   int st = check_shape(M, N, K);
+  if (st == MI355X_FP8_OK) st = check_fast_shape(K);
   if (st != MI355X_FP8_OK) return st;
   if (K > 256 * kStepK) return fail(MI355X_FP8_ENOTSUP, "block-scaled form handles K <= %d (got %lld)",
                                     256 * kStepK, (long long)K);
