@@ -38,19 +38,19 @@
 
 #include "../../include/mi355x_fp8_rowwise.h"
 
-namespace {
-
-typedef int   v4i  __attribute__((ext_vector_type(4)));
-typedef int   v8i  __attribute__((ext_vector_type(8)));
-typedef float v4f  __attribute__((ext_vector_type(4)));
-typedef float v16f __attribute__((ext_vector_type(16)));
-typedef unsigned short us4 __attribute__((ext_vector_type(4)));
-typedef unsigned int v2u __attribute__((ext_vector_type(2)));
-
-constexpr int kNumXcd = 8;       // accelerator complex dies; workgroup ids round-robin over them
-constexpr int kNumCu = 256;
-constexpr int kChunk = 16;       // bytes moved per lane per load
-
+// ------------------------------------------------------------------------------------
+// Building in parts. This file compiles on its own (`hipcc -shared` on it gives the library), and
+// it compiles faster as several translation units in parallel, which is what the package's build
+// script does: with -DMI355X_TILED_PART=<k> a unit holds only the instantiations of tile
+// configuration k of the plain tiled kernel (where nearly all of the compile time goes), with
+// -DMI355X_SPLIT_MAIN it holds everything else and calls those through the functions below.
+// What the units share lives in this namespace (hidden from the library's users): the parameter
+// block, the error text, the table of kernels that need a raised LDS limit, the device set-up.
+// ------------------------------------------------------------------------------------
+#if defined(MI355X_TILED_PART) && defined(MI355X_SPLIT_MAIN)
+#error "a translation unit is either a part or the main unit"
+#endif
+namespace mi355x_shared __attribute__((visibility("hidden"))) {
 struct GemmParams {
   const uint8_t* a;
   const uint8_t* b;
@@ -79,6 +79,42 @@ struct GemmParams {
   // the constant 100 MHz clock (4 values per workgroup), or nullptr
   unsigned long long* stamps;
 };
+
+extern thread_local char err[512];
+struct LdsKernel {
+  const void* kernel;
+  size_t lds_bytes;
+};
+constexpr int kMaxLdsKernels = 256;
+extern LdsKernel lds_kernels[kMaxLdsKernels];
+extern int num_lds_kernels;
+extern bool lds_table_overflow;
+int ready_device(int* dev_out);
+// tile configuration k of the plain tiled kernel: picks the instantiation for the plan in `p` and launches it
+constexpr int kNumTiledParts = 7;
+int tiled_config_0(const GemmParams& p, hipStream_t stream);
+int tiled_config_1(const GemmParams& p, hipStream_t stream);
+int tiled_config_2(const GemmParams& p, hipStream_t stream);
+int tiled_config_3(const GemmParams& p, hipStream_t stream);
+int tiled_config_4(const GemmParams& p, hipStream_t stream);
+int tiled_config_5(const GemmParams& p, hipStream_t stream);
+int tiled_config_6(const GemmParams& p, hipStream_t stream);
+}  // namespace mi355x_shared
+
+namespace {
+
+typedef int   v4i  __attribute__((ext_vector_type(4)));
+typedef int   v8i  __attribute__((ext_vector_type(8)));
+typedef float v4f  __attribute__((ext_vector_type(4)));
+typedef float v16f __attribute__((ext_vector_type(16)));
+typedef unsigned short us4 __attribute__((ext_vector_type(4)));
+typedef unsigned int v2u __attribute__((ext_vector_type(2)));
+
+constexpr int kNumXcd = 8;       // accelerator complex dies; workgroup ids round-robin over them
+constexpr int kNumCu = 256;
+constexpr int kChunk = 16;       // bytes moved per lane per load
+
+using mi355x_shared::GemmParams;
 
 // Where a tile sits: rows [m0, m_end) of A and C it may touch, first column, group.
 struct TileLoc {
@@ -2612,12 +2648,10 @@ __global__ __launch_bounds__(THREADS* ROWS) void fused_rowwise_quant_kernel(cons
 // ------------------------------------------------------------------------------------
 // Host side
 // ------------------------------------------------------------------------------------
-thread_local char g_err[512] = "";
-
 int fail(int code, const char* fmt, ...) {
   va_list ap;
   va_start(ap, fmt);
-  vsnprintf(g_err, sizeof(g_err), fmt, ap);
+  vsnprintf(mi355x_shared::err, sizeof(mi355x_shared::err), fmt, ap);
   va_end(ap);
   return code;
 }
@@ -2647,6 +2681,7 @@ struct TileConfig {
   float wg_stream_share;      // what one workgroup can stream, in units of 1/256 of that rate
 };
 constexpr int kNumTileConfigs = 7;
+static_assert(kNumTileConfigs == mi355x_shared::kNumTiledParts, "one part function per tile configuration");
 constexpr int kDeepSmallConfig = 6;  // 128x128 tiles with three steps in flight, one workgroup per CU
 constexpr int kNumGroupedTileConfigs = 3;  // the grouped form uses the first three
 // Measured on MI355X with normally distributed operands (clock under sustained MFMA load).
@@ -2865,8 +2900,9 @@ inline TiledPlan plan_tiled(int64_t M, int64_t N, int64_t K, int force_config, i
       // (the deep ring takes three steps to fill: short rows of K stay with the two-step form, 2048 x 2048 x 512
       // 6.5 us against 6.9)
       if (c == kDeepSmallConfig && force_config < 0 && sps < 8) continue;
-      // (with one or two tile rows B is fetched with the streaming policy, which this form was not measured
-      // ahead with: 256 x 4096 x 8192 37.7 us against 20.1 for the 64x256 tiles)
+      // (with one or two tile rows the other configurations fetch B with the streaming policy; the deep form with
+      // that policy measured 37.7 us on 256 x 4096 x 8192 against 20.1 for the 64x256 tiles, so it neither has the
+      // policy nor is chosen for such shapes)
       if (c == kDeepSmallConfig && force_config < 0 && M <= 2 * 128) continue;
       const float cost = plan_cost_us(M, N, K, c, splits, sps);
       if (best_cost < 0.0f || cost < best_cost) {
@@ -2906,17 +2942,12 @@ int check_device_shape(int dev) {
 // Setting a device up walks the table once and raises each kernel's limit there, so that no
 // launch path has anything but the launch itself to do: a caller whose first use of some
 // instantiation happens under graph capture meets no attribute call.
-struct LdsKernel {
-  const void* kernel;
-  size_t lds_bytes;
-};
-constexpr int kMaxLdsKernels = 256;
-LdsKernel g_lds_kernels[kMaxLdsKernels];
-int g_num_lds_kernels = 0;
-bool g_lds_table_overflow = false;
+// (The table is shared by the translation units of a build in parts; it is zero-initialised storage,
+// so registrations from any unit's static initialisers find it ready.)
 bool register_lds_kernel(const void* kernel, size_t lds_bytes) {
-  if (g_num_lds_kernels < kMaxLdsKernels) g_lds_kernels[g_num_lds_kernels++] = {kernel, lds_bytes};
-  else g_lds_table_overflow = true;
+  using namespace mi355x_shared;
+  if (num_lds_kernels < mi355x_shared::kMaxLdsKernels) lds_kernels[num_lds_kernels++] = {kernel, lds_bytes};
+  else lds_table_overflow = true;
   return true;
 }
 template <auto Kernel, size_t LdsBytes>
@@ -2926,12 +2957,22 @@ struct LdsLimit {
 
 // 0 = not set up, 1 = ready, -1 = refused (wrong device shape). Setting a device up twice from two
 // threads is harmless: every step is idempotent.
+#if !defined(MI355X_TILED_PART)
 std::atomic<int> g_device_state[kMaxDevices];
 std::atomic<void*> g_scratch_ptr[kMaxDevices];
 int setup_device(int dev);
+#endif
+inline int ready_device(int* dev_out = nullptr) { return mi355x_shared::ready_device(dev_out); }
+}  // namespace
+
+#if !defined(MI355X_TILED_PART)
+thread_local char mi355x_shared::err[512] = "";
+mi355x_shared::LdsKernel mi355x_shared::lds_kernels[mi355x_shared::kMaxLdsKernels];
+int mi355x_shared::num_lds_kernels = 0;
+bool mi355x_shared::lds_table_overflow = false;
 
 // The current device, set up. The only HIP call on the ready path is hipGetDevice.
-int ready_device(int* dev_out = nullptr) {
+int mi355x_shared::ready_device(int* dev_out) {
   int dev = 0;
   const hipError_t e = hipGetDevice(&dev);
   if (e != hipSuccess) return fail(MI355X_FP8_ELAUNCH, "hipGetDevice: %s", hipGetErrorString(e));
@@ -2940,7 +2981,9 @@ int ready_device(int* dev_out = nullptr) {
   if (g_device_state[dev].load(std::memory_order_acquire) == 1) return MI355X_FP8_OK;
   return setup_device(dev);
 }
+#endif
 
+namespace {
 template <int BM, int BN, int WAVES_M, int WAVES_N, bool KTAIL, int EPI, bool GROUPED = false, bool BLOCKSCALE = false,
           int DIST = kDefaultDist, bool STREAM_B = false>
 int launch_tiled(GemmParams p, hipStream_t stream) {
@@ -2996,7 +3039,39 @@ int launch_tiled_config(const GemmParams& p, hipStream_t s) {
   }
   return launch_tiled_epilogue<BM, BN, WAVES_M, WAVES_N, false, DEEP>(p, s);
 }
+}  // namespace
 
+// The seven tile configurations of the plain tiled kernel, each behind a function of its own: a unit
+// of a build in parts defines one of them, the main unit of such a build none, a single-unit build all.
+#if !defined(MI355X_SPLIT_MAIN)
+#define MI355X_DEFINE_TILED_PART(k, ...)                                                             \
+  int mi355x_shared::tiled_config_##k(const GemmParams& p, hipStream_t stream) { return launch_tiled_config<__VA_ARGS__>(p, stream); }
+#if !defined(MI355X_TILED_PART) || MI355X_TILED_PART == 0
+MI355X_DEFINE_TILED_PART(0, 256, 256, 2, 2, true)
+#endif
+#if !defined(MI355X_TILED_PART) || MI355X_TILED_PART == 1
+MI355X_DEFINE_TILED_PART(1, 128, 128, 2, 2, true)
+#endif
+#if !defined(MI355X_TILED_PART) || MI355X_TILED_PART == 2
+MI355X_DEFINE_TILED_PART(2, 256, 128, 2, 2, true)
+#endif
+#if !defined(MI355X_TILED_PART) || MI355X_TILED_PART == 3
+MI355X_DEFINE_TILED_PART(3, 64, 256, 1, 4, true)
+#endif
+#if !defined(MI355X_TILED_PART) || MI355X_TILED_PART == 4
+MI355X_DEFINE_TILED_PART(4, 128, 256, 2, 2, true)
+#endif
+#if !defined(MI355X_TILED_PART) || MI355X_TILED_PART == 5
+MI355X_DEFINE_TILED_PART(5, 192, 256, 2, 2, true)
+#endif
+#if !defined(MI355X_TILED_PART) || MI355X_TILED_PART == 6
+MI355X_DEFINE_TILED_PART(6, 128, 128, 2, 2, false, true)  // (never with the streaming policy)
+#endif
+#undef MI355X_DEFINE_TILED_PART
+#endif
+
+#if !defined(MI355X_TILED_PART)  // (everything from here on belongs to the main unit)
+namespace {
 template <int MT, int NTW, int DEPTH, int KW>
 int launch_skinny(const GemmParams& p, hipStream_t stream) {
   constexpr size_t lds_bytes = (size_t)KW * (NTW + MT) * 16 * kStepK;
@@ -3028,14 +3103,14 @@ int setup_device(int dev) {
   if (g_device_state[dev].load(std::memory_order_acquire) < 0)
     return fail(MI355X_FP8_ENOTSUP, "device %d does not report the %d compute units these kernels are scheduled for "
                 "(a partitioned mode or another part)", dev, kNumCu);
-  if (g_lds_table_overflow) return fail(MI355X_FP8_ELAUNCH, "kernel table overflow (more than %d instantiations)", kMaxLdsKernels);
+  if (mi355x_shared::lds_table_overflow) return fail(MI355X_FP8_ELAUNCH, "kernel table overflow (more than %d instantiations)", mi355x_shared::kMaxLdsKernels);
   if (const int st = check_device_shape(dev)) {
     if (st == MI355X_FP8_ENOTSUP) g_device_state[dev].store(-1, std::memory_order_release);
     return st;
   }
-  for (int i = 0; i < g_num_lds_kernels; ++i) {
-    const hipError_t e = hipFuncSetAttribute(g_lds_kernels[i].kernel, hipFuncAttributeMaxDynamicSharedMemorySize,
-                                             (int)g_lds_kernels[i].lds_bytes);
+  for (int i = 0; i < mi355x_shared::num_lds_kernels; ++i) {
+    const hipError_t e = hipFuncSetAttribute(mi355x_shared::lds_kernels[i].kernel, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                             (int)mi355x_shared::lds_kernels[i].lds_bytes);
     if (e != hipSuccess) return fail(MI355X_FP8_ELAUNCH, "hipFuncSetAttribute: %s", hipGetErrorString(e));
   }
   void* ptr = nullptr;
@@ -3165,7 +3240,7 @@ int mi355x_fp8_rowwise_abi_version(void) { return MI355X_FP8_ABI_VERSION; }
 
 int mi355x_fp8_rowwise_init(void) { return ready_device(); }
 
-const char* mi355x_fp8_rowwise_last_error(void) { return g_err; }
+const char* mi355x_fp8_rowwise_last_error(void) { return mi355x_shared::err; }
 
 int mi355x_fp8_rowwise_select_variant(int64_t M, int64_t N, int64_t K) {
   const int st = check_shape(M, N, K);
@@ -3305,13 +3380,13 @@ int run_gemm(const void* a, const void* b, const float* a_scale, const float* b_
         p.steps_per_split = plan.steps_per_split;
         p.partial = plan.splits > 1 ? (float*)workspace : nullptr;
         switch (plan.config) {
-          case 0: return launch_tiled_config<256, 256, 2, 2, true>(p, s);
-          case 1: return launch_tiled_config<128, 128, 2, 2, true>(p, s);
-          case 2: return launch_tiled_config<256, 128, 2, 2, true>(p, s);
-          case 3: return launch_tiled_config<64, 256, 1, 4, true>(p, s);
-          case 4: return launch_tiled_config<128, 256, 2, 2, true>(p, s);
-          case 5: return launch_tiled_config<192, 256, 2, 2, true>(p, s);
-          case 6: return launch_tiled_config<128, 128, 2, 2, true, true>(p, s);
+          case 0: return mi355x_shared::tiled_config_0(p, s);
+          case 1: return mi355x_shared::tiled_config_1(p, s);
+          case 2: return mi355x_shared::tiled_config_2(p, s);
+          case 3: return mi355x_shared::tiled_config_3(p, s);
+          case 4: return mi355x_shared::tiled_config_4(p, s);
+          case 5: return mi355x_shared::tiled_config_5(p, s);
+          case 6: return mi355x_shared::tiled_config_6(p, s);
           default: return fail(MI355X_FP8_EINVAL, "unknown tile configuration %d", plan.config);
         }
       }
@@ -3633,3 +3708,4 @@ int mi355x_fp8_silu_mul_rowwise_quantize(const void* x1, const void* x2, void* x
 }
 
 }  // extern "C"
+#endif  // !MI355X_TILED_PART
