@@ -3,9 +3,10 @@ alternatives, timed on the device: the cost estimates behind the choice are tabl
 constants, and a table that has drifted away from the kernels shows here as a choice that is
 clearly slower than one of its alternatives. Needs an MI355X.
 
-Timing: a captured graph of 16 launches over 4 rotating operand sets (cold weights, as a model's
-are), best of 4 replays after a warm-up replay. The bar is 12 %: the spread of repeated
-measurements of one plan on these shapes is 2-4 %.
+Timing (tritonbench_amd/tuning.py, the module behind the autotuned backend): a captured graph of
+16 launches over rotating operand sets (cold weights, as a model's are), sustained bursts, the
+median of three. The bar is 12 %: the spread of repeated measurements of one plan on these shapes
+is 2-5 %.
 
 These are wall-clock assertions, not parity: they carry the `perf` marker beside `gpu`
 (`-m "gpu and not perf"` leaves them out), every shape prints its margin, and the file sorts behind
@@ -13,7 +14,7 @@ every parity file so that a noisy replay cannot keep `pytest -x` from reaching t
 import pytest
 import torch
 
-from tritonbench_amd import _lib, ops
+from tritonbench_amd import _lib, tuning
 
 pytestmark = [pytest.mark.gpu, pytest.mark.perf]
 
@@ -38,67 +39,23 @@ SHAPES = [(32, 8192, 8192, False), (64, 8192, 8192, False), (128, 8192, 8192, Fa
           (768, 2048, 2048, False)]
 
 
-def _time_us(dev, m, n, k, bias, variant, sets):
-    ws = ops.gemm_workspace(m, n, k, dev, variant)
-    stream = torch.cuda.Stream()
-    with torch.cuda.stream(stream):
-        def call(i):
-            xq, wq, xs, w_s, b, out = sets[i % len(sets)]
-            ops.fp8_gemm_rowwise(xq, wq, xs, w_s, bias=b, out=out, workspace=ws, variant=variant)
-        call(0)
-        torch.cuda.synchronize()
-        g = torch.cuda.CUDAGraph()
-        with torch.cuda.graph(g, stream=stream):
-            for i in range(16):
-                call(i)
-        g.replay()
-        torch.cuda.synchronize()
-        # Sustained bursts of about 6 ms (as the benchmark times its rows), the median of three: the cost
-        # tables are calibrated on mean step times under sustained load, and short bursts flatter the
-        # candidates that are bound by HBM.
-        def burst(replays):
-            start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-            start.record(stream)
-            for _ in range(replays):
-                g.replay()
-            end.record(stream)
-            torch.cuda.synchronize()
-            return start.elapsed_time(end) * 1e3 / (16 * replays)
-        replays = max(1, int(6000.0 / (16 * max(burst(1), 1.0))))
-        samples = [burst(replays) for _ in range(3)]
-    return sorted(samples)[len(samples) // 2]
-
-
 @pytest.mark.parametrize("m,n,k,bias", SHAPES)
 def test_automatic_choice_is_close_to_the_best_alternative(gpu_device, m, n, k, bias):
     print(f"case m={m} n={n} k={k} bias={bias}", flush=True)
     dev = gpu_device
-    g = torch.Generator(device=dev).manual_seed(m + n + k)
-    sets = []
     # operand sets to rotate through: more than twice the 256 MB memory-side cache in total, as the
     # cost tables are calibrated on operands that come from HBM
-    n_sets = min(10, max(4, 600_000_000 // (n * k) + 1))
-    for _ in range(n_sets):
-        xq, xs = ops.fp8_row_quantize(torch.randn((m, k), generator=g, device=dev))
-        wq, w_s = ops.fp8_row_quantize(torch.randn((n, k), generator=g, device=dev))
-        b = (0.1 * torch.randn((n,), generator=g, device=dev)).to(torch.bfloat16) if bias else None
-        sets.append((xq, wq, xs, w_s, b, torch.empty((m, n), dtype=torch.bfloat16, device=dev)))
-    alternatives = {f"tiled config {c}": _lib.tiled_variant(c, 0) for c in range(_lib.NUM_TILE_CONFIGS)}
-    if m <= 64:
-        alternatives["skinny"] = _lib.VARIANT_SKINNY
-        alternatives["skinny, one tile per workgroup"] = _lib.VARIANT_SKINNY | _lib.SKINNY_ONE_TILE
-    # (the narrow-tile form also takes up to 256 rows where 64x64 tiles are one round of workgroups)
-    if _lib.skinny_family_takes(m, n):
-        alternatives["skinny, narrow tiles"] = _lib.VARIANT_SKINNY | _lib.SKINNY_NARROW
+    sets = tuning.make_operand_sets(m, n, k, bias, dev)
+    alternatives = tuning.candidates(m, n, k)
     # two rounds over all candidates, the automatic choice first and last: whatever is timed first
     # runs on a colder clock
     # (a third round only if the bound does not hold after two: one noisy replay must not fail the suite)
     times, auto = {name: float("inf") for name in alternatives}, float("inf")
     for rnd in range(3):
-        auto = min(auto, _time_us(dev, m, n, k, bias, _lib.VARIANT_AUTO, sets))
+        auto = min(auto, tuning.time_variant_us(sets, _lib.VARIANT_AUTO))
         for name, v in alternatives.items():
-            times[name] = min(times[name], _time_us(dev, m, n, k, bias, v, sets))
-        auto = min(auto, _time_us(dev, m, n, k, bias, _lib.VARIANT_AUTO, sets))
+            times[name] = min(times[name], tuning.time_variant_us(sets, v))
+        auto = min(auto, tuning.time_variant_us(sets, _lib.VARIANT_AUTO))
         if rnd >= 1 and auto <= TOLERANCE * min(times.values()):
             break
     best_name = min(times, key=times.get)

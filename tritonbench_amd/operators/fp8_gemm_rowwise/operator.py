@@ -152,6 +152,22 @@ class Operator(BenchmarkOperator):
         workspace = ops.gemm_workspace(xq.shape[0], wq.shape[0], xq.shape[1], xq.device)
         return lambda: ops.fp8_gemm_rowwise(xq, wq, x_scale, w_scale, bias=bias, out=out, workspace=workspace)
 
+    @register_benchmark(enabled=False, label="hip_mi355x_autotuned")
+    def _hip_mi355x_autotuned(self, xq, wq, x_scale, w_scale, bias) -> Callable:
+        """The same library with the plan chosen by timing every candidate for the shape once (outside
+        the timed callable; cached per shape), the way the reference's Triton kernels are autotuned.
+        Off by default (the sweep costs a second or two per shape): ask for it with --only."""
+        if not xq.is_cuda:
+            raise NotImplementedError("the MI355X backend needs device tensors (run with --device cuda)")
+        from tritonbench_amd import tuning
+
+        m, k = xq.shape
+        n = wq.shape[0]
+        variant, _, _ = tuning.autotune(m, n, k, xq.device, bias=bias is not None)
+        out = torch.empty((m, n), dtype=torch.bfloat16, device=xq.device)
+        workspace = ops.gemm_workspace(m, n, k, xq.device, variant)
+        return lambda: ops.fp8_gemm_rowwise(xq, wq, x_scale, w_scale, bias=bias, out=out, workspace=workspace, variant=variant)
+
     @register_benchmark(baseline=True, label="torch_cpu_ref")
     def _torch_dequant_cpu(self, xq, wq, x_scale, w_scale, bias) -> Callable:
         hx, hw = xq.cpu(), wq.cpu()
