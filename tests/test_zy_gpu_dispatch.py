@@ -5,8 +5,9 @@ clearly slower than one of its alternatives. Needs an MI355X.
 
 Timing (tritonbench_amd/tuning.py, the module behind the autotuned backend): a captured graph of
 16 launches over rotating operand sets (cold weights, as a model's are), sustained bursts, the
-median of three. The bar is 12 %: the spread of repeated measurements of one plan on these shapes
-is 2-5 %.
+median of three. The bar is 15 %: repeated measurements of one and the same plan on the shorter of
+these shapes (10-30 us) differ by up to 8 % within a run (1 x 8192 x 16384 and 2048^3 have both shown
+the automatic choice and the identical pinned plan that far apart).
 
 These are wall-clock assertions, not parity: they carry the `perf` marker beside `gpu`
 (`-m "gpu and not perf"` leaves them out), every shape prints its margin, and the file sorts behind
@@ -18,7 +19,7 @@ from tritonbench_amd import _lib, tuning
 
 pytestmark = [pytest.mark.gpu, pytest.mark.perf]
 
-TOLERANCE = 1.12
+TOLERANCE = 1.15
 # decode- and small-prefill-sized rows of the Llama-3-70B projection sweep, and the small ragged shape with bias
 SHAPES = [(32, 8192, 8192, False), (64, 8192, 8192, False), (128, 8192, 8192, False), (128, 10240, 8192, False),
           (32, 10240, 8192, False), (256, 8192, 8192, False), (1000, 3000, 4112, True),

@@ -1719,14 +1719,19 @@ __global__ __launch_bounds__(512) void gemm_narrow_kernel(GemmParams p) {
   // each other on one XCD (workgroup ids go round the XCDs), so the tile's rows of B come from HBM once
   // and from that XCD's L2 for the others.
   const int row_blocks = (p.M + BM - 1) / BM;
+  // Columns of C a tile owns: BN, or fewer where that deals the columns out evenly over the CUs (the host's
+  // choice, a multiple of 4). Rows of B past them lie outside the tile's descriptor and read as zeros without
+  // a memory access; their products are computed and not stored.
+  const int tile_cols = p.tiles_n;
   int tile = blockIdx.x, row_block = 0;
   if (row_blocks > 1) {
     const int slot = blockIdx.x / kNumXcd;
     row_block = slot % row_blocks;
     tile = (slot / row_blocks) * kNumXcd + (blockIdx.x % kNumXcd);
-    if (tile * BN >= p.N) return;  // (the grid is rounded up to whole rounds of the XCDs)
+    if (tile * tile_cols >= p.N) return;  // (the grid is rounded up to whole rounds of the XCDs)
   }
-  const int n0 = tile * BN, m0 = row_block * BM;
+  const int n0 = tile * tile_cols, m0 = row_block * BM;
+  const int n_end = min(n0 + tile_cols, p.N);
   const int ksteps = (p.K + KS - 1) / KS;  // the last step may be partial (K is a multiple of 16)
   const int rot = (int)(((unsigned)tile * 5u) % (unsigned)ksteps);
   // a lane's 16 bytes of an 8-row group: row lane/8; LDS position lane%8 holds logical chunk
@@ -1859,7 +1864,7 @@ __global__ __launch_bounds__(512) void gemm_narrow_kernel(GemmParams p) {
 #pragma unroll
         for (int w = 1; w < 4; ++w) sum += area[(((w * MB + i) * NB + jb) * 4 + wave) * 64 + lane];
         const int m = m0 + i * 32 + l32, n = nq + 32 * jb;
-        if (m < p.M && n < p.N) {
+        if (m < p.M && n < n_end) {
           float r[4];
 #pragma unroll
           for (int e = 0; e < 4; ++e) {
@@ -1868,13 +1873,13 @@ __global__ __launch_bounds__(512) void gemm_narrow_kernel(GemmParams p) {
           }
           const uint32_t lo = pack_out_x2(r[0], r[1], p.out_f16), hi = pack_out_x2(r[2], r[3], p.out_f16);
           uint16_t* dst = p.c + (size_t)m * p.ldc + n;
-          if (vec && n + 3 < p.N) {
+          if (vec && n + 3 < n_end) {
             *(v2u*)dst = (v2u){lo, hi};
           } else {
             dst[0] = (uint16_t)lo;
-            if (n + 1 < p.N) dst[1] = (uint16_t)(lo >> 16);
-            if (n + 2 < p.N) dst[2] = (uint16_t)hi;
-            if (n + 3 < p.N) dst[3] = (uint16_t)(hi >> 16);
+            if (n + 1 < n_end) dst[1] = (uint16_t)(lo >> 16);
+            if (n + 2 < n_end) dst[2] = (uint16_t)hi;
+            if (n + 3 < n_end) dst[3] = (uint16_t)(hi >> 16);
           }
         }
       }
@@ -1883,7 +1888,7 @@ __global__ __launch_bounds__(512) void gemm_narrow_kernel(GemmParams p) {
     // ---- loader wave for B: slab `wave - 4` of every step, 8 rows per load
     const int w = wave - 4;
     const __amdgpu_buffer_rsrc_t rb = __builtin_amdgcn_make_buffer_rsrc(
-        const_cast<uint8_t*>(p.b) + (size_t)n0 * p.ldb, 0, (int)((uint32_t)min(p.N - n0, BN) * (uint32_t)p.ldb), 0x00020000);
+        const_cast<uint8_t*>(p.b) + (size_t)n0 * p.ldb, 0, (int)((uint32_t)(n_end - n0) * (uint32_t)p.ldb), 0x00020000);
     const uint32_t b_even = (uint32_t)ld_row * (uint32_t)p.ldb + chunk_even;
     const uint32_t b_odd = (uint32_t)ld_row * (uint32_t)p.ldb + (chunk_even ^ 64u);
     auto issue_b = [&](int s) {
@@ -2753,12 +2758,21 @@ inline long narrow_workgroups(int64_t M, int64_t N, NarrowForm f) {
   const long tiles = (N + 32 * f.nb - 1) / (32 * f.nb), row_blocks = (M + 32 * f.mb - 1) / (32 * f.mb);
   return row_blocks == 1 ? tiles : (tiles + kNumXcd - 1) / kNumXcd * kNumXcd * row_blocks;
 }
+// Columns per tile where all rows sit in one workgroup: the columns dealt out evenly over the CUs, in multiples
+// of 4 (8-byte stores), up to the 64 a workgroup can take; beyond 64 x 256 columns the launch needs several
+// rounds of workgroups anyway and the tiles stay 32 wide.
+inline int narrow_tile_cols(int64_t N) {
+  if (N > 64 * (int64_t)kNumCu) return 32;
+  const int64_t per_cu = (N + kNumCu - 1) / kNumCu;
+  const int w = (int)((per_cu + 3) / 4 * 4);
+  return w < 4 ? 4 : w;
+}
 inline NarrowForm narrow_form(int64_t M, int64_t N) {
-  if (M <= 32) return {1, narrow_is_wide(N) ? 2 : 1};
+  if (M <= 32) return {1, narrow_tile_cols(N) > 32 ? 2 : 1};
   static const NarrowForm by_size[3] = {{1, 1}, {2, 1}, {2, 2}};
   for (const NarrowForm f : by_size)
     if (narrow_workgroups(M, N, f) <= kNumCu) return f;
-  return {2, narrow_is_wide(N) ? 2 : 1};  // (M <= 64: several rounds of workgroups)
+  return {2, narrow_tile_cols(N) > 32 ? 2 : 1};  // (M <= 64: all rows in one workgroup)
 }
 inline float narrow_cost_us(int64_t M, int64_t N, int64_t K) {
   const NarrowForm f = narrow_form(M, N);
@@ -2769,11 +2783,16 @@ inline float narrow_cost_us(int64_t M, int64_t N, int64_t K) {
     if (f.mb == 2) return 5.4f + k1024 * (0.75f + 0.575f * share);
     return 3.5f + k1024 * (0.9f + 0.25f * share);
   }
-  // (K = 28672, N = 10240, M = 32: 58.7 us, a lower rate than the shorter rows reach)
-  if (narrow_is_wide(N))
-    // (four 512-byte steps, K = 2048: 7.4 us at 4 x 13312)
-    return M <= 32 ? (K <= 2048 ? 3.0f : 4.0f) + (float)N * (float)K / (K > 16384 ? 5.0e6f : 6.3e6f)
-                   : 8.0f + (float)N * (float)K / (K > 16384 ? 5.5e6f : 7.0e6f);
+  // All rows in one workgroup, one round of workgroups: the columns are dealt out evenly (narrow_tile_cols), and
+  // what a workgroup waits for is its operands against the fetches a CU can have outstanding (about 64 KB): its
+  // rows of B at HBM's latency (2 us), its rows of A at the L2's (0.6 us), plus start and launch. Measured cold at
+  // M = 32, K = 8192: N = 1024 8.5 us, 2048 8.9, 4096 11.9, 5120 11.7, 8192 14.5, 10240 17.2, 16384 23.5 (N = 12288:
+  // 21.1, three more than this says: with 48-column tiles the chip as a whole delivers less); K = 4096: N = 4096 7.3,
+  // 14336 12.9; M = 64: 8192 x 8192 17.9, 10240 x 8192 20.6; M = 16: 13312 x 13312 29.3.
+  if (N <= 64 * (int64_t)kNumCu) {
+    const float w = (float)narrow_tile_cols(N);
+    return 4.4f + w * (float)K / 32768.0f + (float)M * (float)K * (0.6f / 65536.0f);
+  }
   const long tiles = (N + 31) / 32;
   const long rounds = (tiles + kNumCu - 1) / kNumCu;
   // per 1024 bytes of K: what the CUs at work can pull from L2, or, with most of them at work and up to 32
@@ -3211,11 +3230,14 @@ int launch_narrow(const GemmParams& p, hipStream_t stream) {
   constexpr auto kern = gemm_narrow_kernel<MB, NB>;
   (void)LdsLimit<kern, lds_bytes>::registered;
   if (const int st = ready_device()) return st;
-  const unsigned tiles = (unsigned)((p.N + 32 * NB - 1) / (32 * NB));
   const unsigned row_blocks = (unsigned)((p.M + 32 * MB - 1) / (32 * MB));
+  GemmParams q = p;
+  q.tiles_n = row_blocks == 1 ? narrow_tile_cols(p.N) : 32 * NB;  // columns per tile
+  if (q.tiles_n > 32 * NB) return fail(MI355X_FP8_ELAUNCH, "narrow-tile form and tile width disagree");
+  const unsigned tiles = (unsigned)((p.N + q.tiles_n - 1) / q.tiles_n);
   // (with row blocks the kernel deals tiles out per XCD: whole rounds of the XCDs)
   const unsigned grid = row_blocks == 1 ? tiles : (tiles + kNumXcd - 1) / kNumXcd * kNumXcd * row_blocks;
-  hipLaunchKernelGGL(kern, dim3(grid), dim3(512), lds_bytes, stream, p);
+  hipLaunchKernelGGL(kern, dim3(grid), dim3(512), lds_bytes, stream, q);
   hipError_t e = hipGetLastError();
   if (e != hipSuccess) return fail(MI355X_FP8_ELAUNCH, "narrow-tile kernel launch: %s", hipGetErrorString(e));
   return MI355X_FP8_OK;
