@@ -11,16 +11,21 @@
 //                            steps staged global->LDS with direct-to-LDS loads into swizzled
 //                            rings (2 or 3 stages of A, one more of B), 32x32x64 MFMA, epilogue
 //                            turned through LDS into 16-byte row stores. Tiles of 256x256,
-//                            128x128, 256x128, 64x256, 128x256 and 192x256; grouped and block-scaled forms.
+//                            128x128 (two ring depths), 256x128, 64x256, 128x256 and 192x256; grouped
+//                            and block-scaled forms.
 //   splitk_finalize_kernel   adds the fp32 partial sums of a split-K launch, applies scales/bias.
 //   gemm_skinny_kernel       M <= 64: every workgroup owns 16 rows of B and all of K, its waves
 //                            split K between them and reduce through LDS; B is streamed once.
 //   gemm_skinny_persistent_kernel  M <= 16 (M <= 32 at K = 4096): one 16-wave workgroup per CU keeps
 //                            its share of A in registers and walks 16-row tiles of B.
-//   gemm_narrow_kernel       M <= 64 (M <= 256 in row blocks), K in 512-byte steps, at most one 32- or
-//                            64-column tile per CU: a workgroup owns all of K (no split, no second
+//   gemm_skinny_pair_kernel  M <= 16, N <= 8192, K <= 8192: one or two 16-row tiles of B per CU, A parked
+//                            in LDS, a tile's rows requested in one burst.
+//   gemm_narrow_kernel       M <= 64 (M <= 256 in row blocks), K in 512-byte steps, at most one tile of
+//                            up to 64 columns per CU: a workgroup owns all of K (no split, no second
 //                            launch); separate waves fetch A and B.
+//   gemm_generic_kernel      any K, leading dimension and alignment: byte loads, f32 multiply-adds.
 //   quantize_rows_*_kernel   row-wise e4m3fn quantiser (amax, scale, convert), one row per workgroup.
+//   quantize_blocks_kernel   128 x 128 block-wise e4m3fn quantiser, one block per workgroup.
 //   fused_rowwise_quant_kernel  RMSNorm or SiLU-mul of bf16 rows followed by the same quantiser, one pass.
 //
 // Operand roles inside the MFMA are swapped on purpose (rows of B feed the instruction's
@@ -2739,16 +2744,9 @@ inline bool narrow_fits(int64_t M, int64_t N, int64_t K) {
   const long tiles = ((N + 63) / 64 + kNumXcd - 1) / kNumXcd * kNumXcd, row_blocks = (M + 63) / 64;
   return M <= kNarrowMaxM && tiles * row_blocks <= kNumCu;
 }
-// Between one and two 32-column tiles per CU the tiles are 64 columns wide: one round of workgroups on
-// part of the chip instead of two (measured at K = 8192: 18.1 / 19.7 / 23.4 us for N = 10240 / 12288 /
-// 16384 with up to 32 rows of A, 22.8 / 27.2 us for N = 10240 / 16384 with up to 64).
-inline bool narrow_is_wide(int64_t N) {
-  const long tiles = (N + 31) / 32;
-  return tiles > kNumCu && tiles <= 2 * kNumCu;
-}
 // The form for a shape: 32-row blocks of A per workgroup (the rows beyond them go to further row
 // blocks) and 32-column blocks per tile. Up to 32 rows, and up to 64 on panels too wide for row
-// blocks: all rows in one workgroup, 64-column tiles between one and two 32-column tiles per CU.
+// blocks: all rows in one workgroup, tiles of narrow_tile_cols() columns (two blocks from 33 columns up).
 // Otherwise the smallest tile whose row blocks are one round of workgroups: more CUs at work, and
 // less to deliver into each one's LDS.
 struct NarrowForm {
