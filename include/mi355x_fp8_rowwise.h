@@ -76,8 +76,10 @@ extern "C" {
  * the whole launch (one 16-wave workgroup per CU): the pair form for N <= 8192 and any K <= 8192
  * (at most two tiles of B per CU, A parked in LDS, a tile's loads issued in one burst), the
  * persistent form for larger N with K one of 2048, 4096, 6144, 8192 (a run of tiles per CU, A in
- * registers, rolling prefetch; also M <= 32 at K = 4096) - unless the narrow-tile form below is
- * expected to be faster; every other shape runs the general form anyway. */
+ * registers, rolling prefetch; also M <= 32 at K = 4096) - unless the narrow-tile form below or the
+ * general form is expected to be faster (the general form is, by a few per cent, at M <= 8 on most
+ * shapes, and by more where K is far from a multiple of 2048); every other shape runs the general
+ * form anyway. */
 #define MI355X_FP8_SKINNY_ONE_TILE      (1 << 8)
 /* Skinny family only: bit 9 pins the narrow-tile form (one workgroup per 32 or 64 columns of C owns
  * all of K). It takes M <= 64 and, in row blocks of 64 with 64-column tiles, 64 < M <= 256 when

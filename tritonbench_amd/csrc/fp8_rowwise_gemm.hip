@@ -2787,9 +2787,10 @@ inline float narrow_cost_us(int64_t M, int64_t N, int64_t K) {
   // M = 32, K = 8192: N = 1024 8.5 us, 2048 8.9, 4096 11.9, 5120 11.7, 8192 14.5, 10240 17.2, 16384 23.5 (N = 12288:
   // 21.1, three more than this says: with 48-column tiles the chip as a whole delivers less); K = 4096: N = 4096 7.3,
   // 14336 12.9; M = 64: 8192 x 8192 17.9, 10240 x 8192 20.6; M = 16: 13312 x 13312 29.3.
+  // (Fewer than 16 rows of A cost what 16 do: 1 x 5120 x 8192 10.1 us, 16 x 5120 x 8192 10.2.)
   if (N <= 64 * (int64_t)kNumCu) {
     const float w = (float)narrow_tile_cols(N);
-    return 4.4f + w * (float)K / 32768.0f + (float)M * (float)K * (0.6f / 65536.0f);
+    return 4.4f + w * (float)K / 32768.0f + (float)(M < 16 ? 16 : M) * (float)K * (0.6f / 65536.0f);
   }
   const long tiles = (N + 31) / 32;
   const long rounds = (tiles + kNumCu - 1) / kNumCu;
@@ -2801,13 +2802,17 @@ inline float narrow_cost_us(int64_t M, int64_t N, int64_t K) {
   if (M <= 32) return (float)rounds * (3.5f + k1024 * (tiles >= kNumCu / 2 ? fmaxf(1.08f, 1.38f * share) : 1.38f));
   return (float)rounds * (4.5f + k1024 * (1.1f + 0.52f * share));
 }
-inline float skinny_streaming_cost_us(int64_t M, int64_t N, int64_t K) {
-  // the persistent form (measured: 12.7 us at N=K=8192, 71 us at N=57344)
-  // (two blocks of A, K = 4096: 9.9 us at N=8192)
-  // the pair kernel (measured cold: 12.75 us at N=K=8192, 7.9 at K=4096, 5.4 at K=2048; 8.7 at 4096 x 8192, one tile per CU)
-  if (pair_skinny_fits(M, N, K)) return (N <= 16 * kNumCu ? 3.75f : 2.75f) + (float)N * (float)K / 6.7e6f;
-  // (one step per wave, K = 2048: a tile is over before the next one's rows have arrived; 4 x 13312 x 2048 8.2 us)
-  if (persistent_skinny_fits(M, N, K)) return (K <= 2048 ? 4.2f : 3.0f) + (float)N * (float)K / (M <= 16 ? 6.9e6f : 4.9e6f);
+// The pair kernel. Its time follows the CU with the most tiles, and the K steps are dealt to its 16 waves in whole
+// rounds (K = 2304 is 18 steps in 32 slots): half the columns count as dealt evenly, half as the busiest CU's, and K
+// as rounded up to 2048. Measured cold: 16 x 8192 x 8192 12.75 us, K = 4096 7.9, K = 2048 5.4; M = 1: 8192 x 8192
+// 12.4, 4096 x 8192 8.0, 4096 x 4096 5.6, 8192 x 2048 5.1, 4096 x 2304 5.0; M = 16: 5120 x 8192 11.2, 6144 x 8192 11.5.
+inline float pair_cost_us(int64_t N, int64_t K) {
+  const float cols_busiest = (float)(16 * ((N / 16 + kNumCu - 1) / kNumCu) * kNumCu);
+  const float k_slots = (float)((K + 16 * kStepK - 1) / (16 * kStepK) * (16 * kStepK));
+  return (N <= 16 * kNumCu ? 3.1f : 2.75f) + 0.5f * ((float)N + cols_busiest) * k_slots / 6.7e6f;
+}
+// The general kernel, one 16- or 32-row tile of B per workgroup.
+inline float one_tile_cost_us(int64_t M, int64_t N, int64_t K) {
   static const float rate[4] = {6.0e6f, 4.5e6f, 3.44e6f, 3.6e6f};
   const int blocks = (int)((M + 15) / 16);
   const int b = blocks < 1 ? 0 : blocks > 4 ? 3 : blocks - 1;
@@ -2819,15 +2824,33 @@ inline float skinny_streaming_cost_us(int64_t M, int64_t N, int64_t K) {
   // 4096 x 14336 with 256 takes 12.9).
   // (With one or two blocks of A a single round that leaves CUs idle is left as it was: those shapes are a few
   // microseconds long and bound by the launch, 32 x 2048 x 2048 4.5 us.)
-  {
-    const long wgs = (N + (b == 3 ? 31 : 15)) / (b == 3 ? 32 : 16);
-    const long rounds = (wgs + kNumCu - 1) / kNumCu;
-    if (b >= 2 || rounds > 1) r *= (float)wgs / (float)(rounds * kNumCu);
-    // (long rows on part of the chip: a workgroup streams 23 KB per microsecond at most; 32 x 2304 x 16384 takes
-    // 16.2 us with 144 workgroups, 128x128 tiles in splits 14.7)
-    else if (K > 8192 && wgs < kNumCu) r = fminf(r, (float)wgs * 2.35e4f);
+  const long wgs = (N + (b == 3 ? 31 : 15)) / (b == 3 ? 32 : 16);
+  const long rounds = (wgs + kNumCu - 1) / kNumCu;
+  if (b >= 2 || rounds > 1) r *= (float)wgs / (float)(rounds * kNumCu);
+  // (long rows on part of the chip: a workgroup streams 23 KB per microsecond at most; 32 x 2304 x 16384 takes
+  // 16.2 us with 144 workgroups, 128x128 tiles in splits 14.7)
+  else if (K > 8192 && wgs < kNumCu) r = fminf(r, (float)wgs * 2.35e4f);
+  // (up to 16 rows, measured cold: 1 x 8192 x 8192 12.1 us, 1 x 4096 x 8192 7.5, 1 x 2304 x 2048 3.7,
+  // 16 x 8192 x 8192 13.8, 16 x 4096 x 4096 5.6)
+  // (two blocks: 32 x 2048 x 2048 4.5 us)
+  return (b == 0 ? 3.0f : b == 1 ? 3.7f : 5.0f) + (float)N * (float)K / r;
+}
+// The streaming members of the family and which of them runs a shape: the pair kernel where it fits, unless the
+// one-tile kernel is expected ahead (at M <= 8 by a few per cent on most shapes, by 15-20 % where K fills the pair
+// kernel's step slots badly: 1 x 4096 x 2304 4.3 us against 5.0); the persistent kernel beyond the pair kernel's N.
+enum SkinnyStreaming { kStreamPair, kStreamPersistent, kStreamOneTile };
+inline SkinnyStreaming skinny_streaming_choice(int64_t M, int64_t N, int64_t K) {
+  if (pair_skinny_fits(M, N, K)) return one_tile_cost_us(M, N, K) < pair_cost_us(N, K) ? kStreamOneTile : kStreamPair;
+  return persistent_skinny_fits(M, N, K) ? kStreamPersistent : kStreamOneTile;
+}
+inline float skinny_streaming_cost_us(int64_t M, int64_t N, int64_t K) {
+  switch (skinny_streaming_choice(M, N, K)) {
+    case kStreamPair: return pair_cost_us(N, K);
+    // the persistent form (measured: 71 us at 16 x 57344 x 8192; two blocks of A, K = 4096: 9.9 us at N = 8192, 8.9 at
+    // 24 x 6144 x 4096; one step per wave, K = 2048: a tile is over before the next one's rows have arrived, 4 x 13312 x 2048 8.2 us)
+    case kStreamPersistent: return (K <= 2048 ? 4.2f : 3.0f) + (float)N * (float)K / (M <= 16 ? 6.9e6f : 4.4e6f);
+    default: return one_tile_cost_us(M, N, K);
   }
-  return 5.0f + (float)N * (float)K / r;
 }
 // the cheapest member of the M <= 64 family: streaming (persistent or one tile per workgroup) or narrow tiles
 inline bool narrow_preferred(int64_t M, int64_t N, int64_t K) {
@@ -2885,7 +2908,8 @@ inline float plan_cost_us(int64_t M, int64_t N, int64_t K, int config, int split
   // (64x256 tiles, unsplit: the rotated K order lifts the rate further; with two splits the plan measured at the
   // plain rate, 48 x 28672 x 8192 47.5 us)
   // (256x256 tiles gain the most: their rate without the policy is the lowest)
-  const float policy = !streams_b ? 1.0f : (config == 3 && splits == 1) ? 1.08f * 1.1f : config == 0 ? 1.2f : 1.08f;
+  const float policy = !streams_b || config == kDeepSmallConfig ? 1.0f
+                       : (config == 3 && splits == 1) ? 1.08f * 1.1f : config == 0 ? 1.2f : 1.08f;
   // (128x128 tiles: the rate was measured with full tiles; rows of a tile past M are not fetched, and what a CU
   // has to take in beside its rows of B shrinks with them: 64 x 28672 x 8192 unsplit 42.4 us = 6.3 MB/us)
   const float rows_a = (float)M / (float)((M + c.bm - 1) / c.bm);
@@ -2917,10 +2941,13 @@ inline TiledPlan plan_tiled(int64_t M, int64_t N, int64_t K, int force_config, i
       // (the deep ring takes three steps to fill: short rows of K stay with the two-step form, 2048 x 2048 x 512
       // 6.5 us against 6.9)
       if (c == kDeepSmallConfig && force_config < 0 && sps < 8) continue;
-      // (with one or two tile rows the other configurations fetch B with the streaming policy; the deep form with
-      // that policy measured 37.7 us on 256 x 4096 x 8192 against 20.1 for the 64x256 tiles, so it neither has the
-      // policy nor is chosen for such shapes)
-      if (c == kDeepSmallConfig && force_config < 0 && M <= 2 * 128) continue;
+      // (With one or two tile rows the other configurations fetch B with the streaming policy; the deep form with
+      // that policy measured 37.7 us on 256 x 4096 x 8192 against 20.1 for the 64x256 tiles, so it does not have it.
+      // Without it B's lines stay in the caches: on weights small enough to be found there again it is the fastest
+      // plan of all at 96 to 256 rows (operands from the memory-side cache: 256 x 6144 x 4096 14.6 us against 23.8,
+      // 128 x 13312 x 2048 10.0 against 13.9; from HBM level with the 128x128 form), on large ones the policy wins
+      // (64 x 28672 x 8192 from HBM: 51.7 us against 42.7).)
+      if (c == kDeepSmallConfig && force_config < 0 && M <= 2 * 128 && N * K > (int64_t)48 << 20) continue;
       const float cost = plan_cost_us(M, N, K, c, splits, sps);
       if (best_cost < 0.0f || cost < best_cost) {
         best_cost = cost;
@@ -3434,10 +3461,12 @@ int run_gemm(const void* a, const void* b, const float* a_scale, const float* b_
         // 16-byte loads of b_scale, 8-byte loads of bias and 8-byte stores of C when everything is aligned for them
         const bool vec = (reinterpret_cast<uintptr_t>(b_scale) & 15) == 0 && (reinterpret_cast<uintptr_t>(bias) & 7) == 0 &&
                          (reinterpret_cast<uintptr_t>(c) & 7) == 0 && (ldc & 3) == 0;
+        // (pinned, the forms that keep A on chip run wherever they fit; left to the library, where they are expected ahead)
+        const bool resident = (plan_bits & MI355X_FP8_SKINNY_RESIDENT) || skinny_streaming_choice(M, N, K) != kStreamOneTile;
         // (the pair kernel addresses a workgroup's rows of B with 32-bit offsets below 2^31)
-        if (pair_skinny_fits(M, N, K) && ldb * 32 <= (int64_t)INT32_MAX)
+        if (resident && pair_skinny_fits(M, N, K) && ldb * 32 <= (int64_t)INT32_MAX)
           return vec ? launch_skinny_pair_form<true>(p, s) : launch_skinny_pair_form<false>(p, s);
-        if (persistent_skinny_fits(M, N, K))
+        if (resident && persistent_skinny_fits(M, N, K))
           return vec ? launch_skinny_persistent_steps<true>(p, s) : launch_skinny_persistent_steps<false>(p, s);
       }
       if (M <= 16) return launch_skinny<1, 1, 4, 8>(p, s);
