@@ -2790,7 +2790,13 @@ inline float narrow_cost_us(int64_t M, int64_t N, int64_t K) {
   // (Fewer than 16 rows of A cost what 16 do: 1 x 5120 x 8192 10.1 us, 16 x 5120 x 8192 10.2.)
   if (N <= 64 * (int64_t)kNumCu) {
     const float w = (float)narrow_tile_cols(N);
-    return 4.4f + w * (float)K / 32768.0f + (float)(M < 16 ? 16 : M) * (float)K * (0.6f / 65536.0f);
+    // (Narrow panels: with 4 to 16 columns a workgroup there is little to fetch, and what a step of K costs is its
+    // trip to memory against the depth of the ring, 0.07 to 0.1 us per 128 bytes. Up to 16 rows, N = 2048: 5.8 / 8.3 /
+    // 11.8 / 21.8 us at K = 4096 / 8192 / 13312 / 28672; N = 1024 5.7 / 8.2 / - / 20.6, 3072 6.1 / 8.9 / 12.6 / 23.7;
+    // 32 rows, K = 28672: N = 1024 21.7, 2048 23.4, 3072 26.0, 3584 28.8.)
+    const float rows = (float)(M < 16 ? 16 : M);
+    return fmaxf(4.4f + w * (float)K / 32768.0f + rows * (float)K * (0.6f / 65536.0f),
+                 3.2f + (float)K * (5.0e-4f + 0.135e-4f * w + 0.035e-4f * rows));
   }
   const long tiles = (N + 31) / 32;
   const long rounds = (tiles + kNumCu - 1) / kNumCu;
@@ -2806,10 +2812,15 @@ inline float narrow_cost_us(int64_t M, int64_t N, int64_t K) {
 // rounds (K = 2304 is 18 steps in 32 slots): half the columns count as dealt evenly, half as the busiest CU's, and K
 // as rounded up to 2048. Measured cold: 16 x 8192 x 8192 12.75 us, K = 4096 7.9, K = 2048 5.4; M = 1: 8192 x 8192
 // 12.4, 4096 x 8192 8.0, 4096 x 4096 5.6, 8192 x 2048 5.1, 4096 x 2304 5.0; M = 16: 5120 x 8192 11.2, 6144 x 8192 11.5.
-inline float pair_cost_us(int64_t N, int64_t K) {
+// With one tile a CU there is little of B to hide the fetch of A behind (N = 2048, K = 8192: 6.8 us with one row of A,
+// 7.8 with 16; K = 4096: 5.1 / 5.5; N = 8192, K = 8192: 12.4 / 12.75).
+inline float pair_cost_us(int64_t M, int64_t N, int64_t K) {
   const float cols_busiest = (float)(16 * ((N / 16 + kNumCu - 1) / kNumCu) * kNumCu);
   const float k_slots = (float)((K + 16 * kStepK - 1) / (16 * kStepK) * (16 * kStepK));
-  return (N <= 16 * kNumCu ? 3.1f : 2.75f) + 0.5f * ((float)N + cols_busiest) * k_slots / 6.7e6f;
+  const float a_rows = N <= 16 * kNumCu ? (float)M * (float)K * (1.1e-4f / 16.0f) : 0.0f;
+  // (a quarter of the CUs at work: 1 x 1024 x 4096 4.95 us, 1 x 1024 x 8192 6.5)
+  const float fixed = N <= 1536 ? 3.35f : N <= 16 * kNumCu ? 3.1f : 2.75f;
+  return fixed + 0.5f * ((float)N + cols_busiest) * k_slots / 6.7e6f + a_rows;
 }
 // The general kernel, one 16- or 32-row tile of B per workgroup.
 inline float one_tile_cost_us(int64_t M, int64_t N, int64_t K) {
@@ -2827,25 +2838,30 @@ inline float one_tile_cost_us(int64_t M, int64_t N, int64_t K) {
   const long wgs = (N + (b == 3 ? 31 : 15)) / (b == 3 ? 32 : 16);
   const long rounds = (wgs + kNumCu - 1) / kNumCu;
   if (b >= 2 || rounds > 1) r *= (float)wgs / (float)(rounds * kNumCu);
-  // (long rows on part of the chip: a workgroup streams 23 KB per microsecond at most; 32 x 2304 x 16384 takes
-  // 16.2 us with 144 workgroups, 128x128 tiles in splits 14.7)
-  else if (K > 8192 && wgs < kNumCu) r = fminf(r, (float)wgs * 2.35e4f);
   // (up to 16 rows, measured cold: 1 x 8192 x 8192 12.1 us, 1 x 4096 x 8192 7.5, 1 x 2304 x 2048 3.7,
   // 16 x 8192 x 8192 13.8, 16 x 4096 x 4096 5.6)
   // (two blocks: 32 x 2048 x 2048 4.5 us)
-  return (b == 0 ? 3.0f : b == 1 ? 3.7f : 5.0f) + (float)N * (float)K / r;
+  float t = (b == 0 ? 3.0f : b == 1 ? 3.7f : 5.0f) + (float)N * (float)K / r;
+  // Part of the chip at work, up to 32 rows: a workgroup has its CU to itself, and a byte of K costs it what its 16
+  // rows of B (from HBM) and its rows of A (from L2) take against the fetches a CU can have outstanding, whatever
+  // the number of workgroups. Measured with 128 workgroups (N = 2048) at K = 4096 / 8192 / 16384 / 28672: one row of
+  // A 4.5 / 6.2 / 9.7 / 14.9 us, 8 rows 4.7 / 6.6 / 10.6 / 17.0, 16 rows 5.1 / 7.6 / 12.2 / 20.5, 32 rows 6.2 / 9.8 /
+  // - / -; with 64 (N = 1024): one row 4.2 / 6.0 / 8.8 / 13.8, 16 rows 4.9 / 7.1 / 11.6 / 19.3; 144 workgroups,
+  // K = 16384: 10.8 / 12.5 / 16.4 us with 8 / 16 / 32 rows.
+  if (b <= 1 && wgs < kNumCu) t = fmaxf(t, 2.6f + (float)K * (4.1e-4f + 0.13e-4f * (float)M));
+  return t;
 }
 // The streaming members of the family and which of them runs a shape: the pair kernel where it fits, unless the
 // one-tile kernel is expected ahead (at M <= 8 by a few per cent on most shapes, by 15-20 % where K fills the pair
 // kernel's step slots badly: 1 x 4096 x 2304 4.3 us against 5.0); the persistent kernel beyond the pair kernel's N.
 enum SkinnyStreaming { kStreamPair, kStreamPersistent, kStreamOneTile };
 inline SkinnyStreaming skinny_streaming_choice(int64_t M, int64_t N, int64_t K) {
-  if (pair_skinny_fits(M, N, K)) return one_tile_cost_us(M, N, K) < pair_cost_us(N, K) ? kStreamOneTile : kStreamPair;
+  if (pair_skinny_fits(M, N, K)) return one_tile_cost_us(M, N, K) < pair_cost_us(M, N, K) ? kStreamOneTile : kStreamPair;
   return persistent_skinny_fits(M, N, K) ? kStreamPersistent : kStreamOneTile;
 }
 inline float skinny_streaming_cost_us(int64_t M, int64_t N, int64_t K) {
   switch (skinny_streaming_choice(M, N, K)) {
-    case kStreamPair: return pair_cost_us(N, K);
+    case kStreamPair: return pair_cost_us(M, N, K);
     // the persistent form (measured: 71 us at 16 x 57344 x 8192; two blocks of A, K = 4096: 9.9 us at N = 8192, 8.9 at
     // 24 x 6144 x 4096; one step per wave, K = 2048: a tile is over before the next one's rows have arrived, 4 x 13312 x 2048 8.2 us)
     case kStreamPersistent: return (K <= 2048 ? 4.2f : 3.0f) + (float)N * (float)K / (M <= 16 ? 6.9e6f : 4.4e6f);
@@ -3296,12 +3312,14 @@ int mi355x_fp8_rowwise_select_variant(int64_t M, int64_t N, int64_t K) {
   // M <= 64: the streaming kernel, unless a tiled plan (64- or 128-row tiles that stream B, split
   // K where the tiles are few) is expected to beat it: from two 16-row blocks of A up on most
   // shapes, with one block on the longest weight panels. Up to 8 rows the streaming kernel was
-  // never behind on any measured shape, so there the estimates are not consulted.
+  // behind on one kind of shape only, few columns with very long rows, where a handful of workgroups
+  // each stream a long tile and split tiles put the whole chip to work (8 x 1024 x 28672: 16.2 us
+  // against 14.5); there a tiled plan has to be expected ahead by a tenth to be taken.
   // (above 64 rows the family's only member is the narrow-tile kernel in row blocks, where it fits)
   if (M > kSkinnyMaxM && !narrow_fits(M, N, K)) return MI355X_FP8_VARIANT_TILED;
-  if (M <= 8) return MI355X_FP8_VARIANT_SKINNY;
-  return plan_tiled(M, N, K, -1, 0, kMaxSplits).cost_us < skinny_cost_us(M, N, K) ? MI355X_FP8_VARIANT_TILED
-                                                                                 : MI355X_FP8_VARIANT_SKINNY;
+  const float margin = M <= 8 ? 0.9f : 1.0f;
+  return plan_tiled(M, N, K, -1, 0, kMaxSplits).cost_us < margin * skinny_cost_us(M, N, K) ? MI355X_FP8_VARIANT_TILED
+                                                                                          : MI355X_FP8_VARIANT_SKINNY;
 }
 
 size_t mi355x_fp8_rowwise_workspace_bytes(int64_t M, int64_t N, int64_t K, int variant) {
