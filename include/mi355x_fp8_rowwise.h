@@ -81,8 +81,8 @@ extern "C" {
  * shapes, and by more where K is far from a multiple of 2048); every other shape runs the general
  * form anyway. */
 #define MI355X_FP8_SKINNY_ONE_TILE      (1 << 8)
-/* Skinny family only: bit 9 pins the narrow-tile form (one workgroup per 32 or 64 columns of C owns
- * all of K). It takes M <= 64 and, in row blocks of 64 with 64-column tiles, 64 < M <= 256 when
+/* Skinny family only: bit 9 pins the narrow-tile form (one workgroup per tile of 4 to 64 columns of C,
+ * the columns dealt out evenly over the CUs, owns all of K). It takes M <= 64 and, in row blocks of 64 with 64-column tiles, 64 < M <= 256 when
  * ceil(M/64) * ceil(N/64, rounded up to a multiple of 8) <= 256 (one workgroup per CU); "not
  * supported" otherwise. Without a pin the family runs whichever of its forms is expected to be
  * fastest. */
