@@ -59,6 +59,10 @@ def time_variant_us(sets: Sequence[OperandSet], variant: int, burst_us: float = 
     n = wq0.shape[0]
     dev = xq0.device
     ws = ops.gemm_workspace(m, n, k, dev, variant)
+    # A fresh stream per call, on purpose: the time of a launch depends on the hardware queue its stream
+    # is mapped to (one captured graph replayed on consecutively created streams: 12.2 / 11.5 / 12.2 /
+    # 13.2 us per launch of 8 x 3072 x 16384, and the same again on the next four), so callers that take
+    # the best of several calls see every plan on several queues.
     stream = torch.cuda.Stream(device=dev)
     with torch.cuda.stream(stream):
         def call(i):
