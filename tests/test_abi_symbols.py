@@ -55,6 +55,11 @@ def test_host_side_argument_checks_need_no_gpu():
         if not _lib.skinny_family_takes(m, n):
             assert lib.mi355x_fp8_rowwise_select_variant(m, n, 1024) == _lib.VARIANT_TILED
     assert lib.mi355x_fp8_rowwise_select_variant(64, 57344, 8192) == _lib.VARIANT_TILED
+    # up to 8 rows the streaming family keeps the shape unless split tiles are expected a tenth ahead
+    # (few columns, very long rows: a handful of workgroups each streaming a long tile)
+    assert lib.mi355x_fp8_rowwise_select_variant(8, 8192, 8192) == _lib.VARIANT_SKINNY
+    assert lib.mi355x_fp8_rowwise_select_variant(1, 2048, 28672) == _lib.VARIANT_SKINNY
+    assert lib.mi355x_fp8_rowwise_select_variant(8, 1024, 28672) == _lib.VARIANT_TILED
     assert lib.mi355x_fp8_rowwise_select_variant(0, 8, 16) == _lib.EINVAL
     assert lib.mi355x_fp8_rowwise_select_variant(8, 8, 24) == _lib.VARIANT_GENERIC  # K not a multiple of 16
     assert lib.mi355x_fp8_rowwise_workspace_bytes(128, 8192, 8200, _lib.VARIANT_AUTO) == 0
