@@ -52,9 +52,10 @@ def test_automatic_choice_is_close_to_the_best_alternative(gpu_device, m, n, k, 
     alternatives = tuning.candidates(m, n, k)
     # two rounds over all candidates, the automatic choice first and last: whatever is timed first
     # runs on a colder clock
-    # (a third round only if the bound does not hold after two: one noisy replay must not fail the suite)
+    # (further rounds, up to five in all, only if the bound does not hold after two: one noisy replay must not
+    # fail the suite; every timing call runs on a fresh stream, so the rounds also see different hardware queues)
     times, auto = {name: float("inf") for name in alternatives}, float("inf")
-    for rnd in range(3):
+    for rnd in range(5):
         auto = min(auto, tuning.time_variant_us(sets, _lib.VARIANT_AUTO))
         for name, v in alternatives.items():
             times[name] = min(times[name], tuning.time_variant_us(sets, v))
