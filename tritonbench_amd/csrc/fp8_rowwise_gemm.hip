@@ -2909,8 +2909,15 @@ inline float plan_cost_us(int64_t M, int64_t N, int64_t K, int config, int split
   const long items = tiles * splits;
   const long slots = (long)kNumCu * c.wgs_per_cu;
   const long full_rounds = items / slots, rest = items % slots;
-  float t = full_rounds * (sps * c.us_per_step + c.us_per_item);
-  if (rest) t += sps * (rest <= kNumCu ? c.us_per_step_alone : c.us_per_step) + c.us_per_item;
+  // (256x128 tiles are bound by the delivery of their operands, and rows of a tile past M are not fetched: with a last
+  // tile row that is half empty a step takes less, 384 x 16384 x 16384 106.5 us = 0.79 us per step instead of 0.87,
+  // 384 x 13312 x 13312 85.7, 640 x 8192 x 8192 53.5, 448 x 10240 x 8192 51.4 where three splits of 256x256 tiles take
+  // 62.8. Unsplit plans only: with the same allowance split plans were taken where they measure behind, 448 x 2304 x
+  // 13312 in seven 33.0 us against 28.5 for the deep 128x128 form in three.)
+  const float rows_fetched = (float)M / (float)((M + c.bm - 1) / c.bm);
+  const float step_scale = config == 2 && splits == 1 ? 0.5f + 0.5f * (rows_fetched + (float)c.bn) / (float)(c.bm + c.bn) : 1.0f;
+  float t = full_rounds * (sps * c.us_per_step * step_scale + c.us_per_item);
+  if (rest) t += sps * (rest <= kNumCu ? c.us_per_step_alone : c.us_per_step) * step_scale + c.us_per_item;
   // (the deep 128x128 form is for one round only; beyond 128 workgroups its steps slow down with the chip's
   // clock and the shared L2: 0.49 us with 128, 0.58 with 256)
   if (config == kDeepSmallConfig) {
