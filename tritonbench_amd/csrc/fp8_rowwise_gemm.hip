@@ -2776,8 +2776,9 @@ inline float narrow_cost_us(int64_t M, int64_t N, int64_t K) {
   const NarrowForm f = narrow_form(M, N);
   if (M > 32 * f.mb) {  // row blocks, one round
     const float k1024 = (float)K / 1024.0f;
-    if (f.nb == 2) return 6.0f + k1024 * (K > 16384 ? 2.15f : 1.9f);
     const float share = (float)narrow_workgroups(M, N, f) / (float)kNumCu;  // of the CUs at work
+    // (64x64 tiles: 1.9 us per 1024 bytes of K with every CU at work, 1.7 with 160 of them, 256 x 2304 x 6656 17.0 us)
+    if (f.nb == 2) return 6.0f + k1024 * (K > 16384 ? 2.15f : 1.34f + 0.56f * share);
     if (f.mb == 2) return 5.4f + k1024 * (0.75f + 0.575f * share);
     return 3.5f + k1024 * (0.9f + 0.25f * share);
   }
