@@ -2849,7 +2849,13 @@ inline float one_tile_cost_us(int64_t M, int64_t N, int64_t K) {
   // A 4.5 / 6.2 / 9.7 / 14.9 us, 8 rows 4.7 / 6.6 / 10.6 / 17.0, 16 rows 5.1 / 7.6 / 12.2 / 20.5, 32 rows 6.2 / 9.8 /
   // - / -; with 64 (N = 1024): one row 4.2 / 6.0 / 8.8 / 13.8, 16 rows 4.9 / 7.1 / 11.6 / 19.3; 144 workgroups,
   // K = 16384: 10.8 / 12.5 / 16.4 us with 8 / 16 / 32 rows.
-  if (b <= 1 && wgs < kNumCu) t = fmaxf(t, 2.6f + (float)K * (4.1e-4f + 0.13e-4f * (float)M));
+  // (Rows that do not start on a 128-byte boundary: every 128-byte piece of a row lies across two cache lines, and a
+  // workgroup alone on its CU, which asks for its rows 128 bytes at a time, takes 1.4-1.5 times as long per byte of K:
+  // 17 x 2816 x 18832 23.6 us where aligned rows would take 15.5, 14 x 1536 x 9760 11.4 against 8.4; the narrow-tile
+  // kernel, 512 bytes of a row at a time, loses 0-12 % on the same shapes. With several rounds of workgroups every
+  // kernel loses about the same, 1.25-1.4, and the order of the estimates holds. K stands in for the row pitch.)
+  const float pitch = K % kStepK != 0 ? 1.45f : 1.0f;
+  if (b <= 1 && wgs < kNumCu) t = fmaxf(t, 2.6f + pitch * (float)K * (4.1e-4f + 0.13e-4f * (float)M));
   return t;
 }
 // The streaming members of the family and which of them runs a shape: the pair kernel where it fits, unless the
