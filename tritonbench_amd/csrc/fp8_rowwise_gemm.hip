@@ -2702,7 +2702,9 @@ constexpr TileConfig kTileConfigs[kNumTileConfigs] = {
     {64, 256, tiled_wgs_per_cu(64, 256), 0.75f, 0.75f, 9.0f, 5.7e6f, 1.42f},
     // (one tile row against a wide panel: 128 x 57344 x 8192 75.2 us with 224 tiles, bound by the stream rate;
     // several tile rows: 512 x 16384 x 16384 125 us with 256 tiles, 4096 x 5120 x 13824 269 us with 640)
-    {128, 256, tiled_wgs_per_cu(128, 256), 0.90f, 0.90f, 10.0f, 5.8e6f, 1.42f},
+    // (a step and a tile's refill and epilogue, from launches that are not bound by the stream rate: 4096 x 2048 x 2048
+    // 18.1 us with 256 tiles of 16 steps, 636 x 12288 x 6144 50.3 with 240 of 48, 512 x 16384 x 16384 125 with 256 of 128)
+    {128, 256, tiled_wgs_per_cu(128, 256), 0.97f, 0.97f, 2.6f, 5.8e6f, 1.42f},
     // (panels whose 256-column tiles come to more than half a round with 256 rows each but fit one with 192:
     // 1024 x 10240 x 8192 73.3 us with 240 tiles, 2048 x 10240 x 8192 135.4 us with 440)
     // (one tile row against a wide panel: 192 x 57344 x 8192 89.2 us)
@@ -2856,6 +2858,9 @@ inline float one_tile_cost_us(int64_t M, int64_t N, int64_t K) {
   // kernel loses about the same, 1.25-1.4, and the order of the estimates holds. K stands in for the row pitch.)
   const float pitch = K % kStepK != 0 ? 1.45f : 1.0f;
   if (b <= 1 && wgs < kNumCu) t = fmaxf(t, 2.6f + pitch * (float)K * (4.1e-4f + 0.13e-4f * (float)M));
+  // (three blocks of A, the same way: 48 x 2048 x 4096 7.5-8.0 us, 48 x 2048 x 8192 12.1-12.6, 34 x 2048 x 1024 3.4,
+  // 48 x 3584 x 28672 36.8; the rate above, scaled by the share of the CUs at work, has these shapes a quarter slower)
+  if (b == 2 && wgs < kNumCu) t = fminf(t, 3.0f + 1.08f * pitch * (float)K * (4.1e-4f + 0.13e-4f * (float)M));
   return t;
 }
 // The streaming members of the family and which of them runs a shape: the pair kernel where it fits, unless the
