@@ -2708,6 +2708,7 @@ constexpr TileConfig kTileConfigs[kNumTileConfigs] = {
     // (panels whose 256-column tiles come to more than half a round with 256 rows each but fit one with 192:
     // 1024 x 10240 x 8192 73.3 us with 240 tiles, 2048 x 10240 x 8192 135.4 us with 440)
     // (one tile row against a wide panel: 192 x 57344 x 8192 89.2 us)
+    // (one round of tiles costs 7 us beside its steps, not 9: plan_cost_us has it)
     {192, 256, tiled_wgs_per_cu(192, 256), 1.00f, 1.00f, 9.0f, 4.9e6f, 1.42f},
     // 128x128 tiles with loads three steps ahead (112 KB of LDS: one workgroup per CU), for launches of at most
     // one workgroup per CU, where a CU has one wave per SIMD and nothing but the depth of the ring to cover
@@ -2928,8 +2929,13 @@ inline float plan_cost_us(int64_t M, int64_t N, int64_t K, int config, int split
   // 13312 in seven 33.0 us against 28.5 for the deep 128x128 form in three.)
   const float rows_fetched = (float)M / (float)((M + c.bm - 1) / c.bm);
   const float step_scale = config == 2 && splits == 1 ? 0.5f + 0.5f * (rows_fetched + (float)c.bn) / (float)(c.bm + c.bn) : 1.0f;
-  float t = full_rounds * (sps * c.us_per_step * step_scale + c.us_per_item);
-  if (rest) t += sps * (rest <= kNumCu ? c.us_per_step_alone : c.us_per_step) * step_scale + c.us_per_item;
+  // (192x256 tiles in a single round: 4712 x 2048 x 1024 14.0-14.8 us with 200 tiles of 8 steps, 416 x 21312 x 1024 15.0
+  // with 252, 2560 x 8192 x 1024 26.6 with 448 where 128x256 tiles take 30.3; over several rounds the table's 9 us per
+  // tile stands: it leaves the estimate as far above the measurement as that of the 256x256 tiles, 3-4 %, and the order
+  // of the two right: 896 x 57344 x 8192 343 us with 256x256 tiles, 354 with these)
+  const float us_per_item = config == 5 && items <= 2 * slots ? 7.0f : c.us_per_item;
+  float t = full_rounds * (sps * c.us_per_step * step_scale + us_per_item);
+  if (rest) t += sps * (rest <= kNumCu ? c.us_per_step_alone : c.us_per_step) * step_scale + us_per_item;
   // (the deep 128x128 form is for one round only; beyond 128 workgroups its steps slow down with the chip's
   // clock and the shared L2: 0.49 us with 128, 0.58 with 256)
   if (config == kDeepSmallConfig) {
