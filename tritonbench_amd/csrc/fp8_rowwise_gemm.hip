@@ -2846,6 +2846,10 @@ inline float one_tile_cost_us(int64_t M, int64_t N, int64_t K) {
   // 16 x 8192 x 8192 13.8, 16 x 4096 x 4096 5.6)
   // (two blocks: 32 x 2048 x 2048 4.5 us)
   float t = (b == 0 ? 3.0f : b == 1 ? 3.7f : 5.0f) + (float)N * (float)K / r;
+  // (Wide panels with short rows: every workgroup has a start and an end that no other hides, 1.7 ns apiece beyond the
+  // first 512, which shows where a workgroup's share of K is short: 3 x 45376 x 1024 14.7 us for 46 MB, 1 x 103104 x
+  // 1664 38.1 for 172 MB, 3 x 97728 x 2304 44.6; at K = 8192 half of it is left, 1 x 57344 x 8192 71.5.)
+  if (b == 0 && wgs > 2 * kNumCu) t += (float)(wgs - 2 * kNumCu) * 1.66e-3f * fminf(1.0f, 4096.0f / (float)K);
   // Part of the chip at work, up to 32 rows: a workgroup has its CU to itself, and a byte of K costs it what its 16
   // rows of B (from HBM) and its rows of A (from L2) take against the fetches a CU can have outstanding, whatever
   // the number of workgroups. Measured with 128 workgroups (N = 2048) at K = 4096 / 8192 / 16384 / 28672: one row of
@@ -2877,7 +2881,10 @@ inline float skinny_streaming_cost_us(int64_t M, int64_t N, int64_t K) {
     case kStreamPair: return pair_cost_us(M, N, K);
     // the persistent form (measured: 71 us at 16 x 57344 x 8192; two blocks of A, K = 4096: 9.9 us at N = 8192, 8.9 at
     // 24 x 6144 x 4096; one step per wave, K = 2048: a tile is over before the next one's rows have arrived, 4 x 13312 x 2048 8.2 us)
-    case kStreamPersistent: return (K <= 2048 ? 4.2f : 3.0f) + (float)N * (float)K / (M <= 16 ? 6.9e6f : 4.4e6f);
+    // (K = 2048, one step per wave: 1 x 128256 x 2048 50.6 us, 4 x 13312 x 2048 8.2)
+    case kStreamPersistent:
+      if (K <= 2048 && M <= 16) return 3.4f + (float)N * (float)K / 5.7e6f;
+      return (K <= 2048 ? 4.2f : 3.0f) + (float)N * (float)K / (M <= 16 ? 6.9e6f : 4.4e6f);
     default: return one_tile_cost_us(M, N, K);
   }
 }
@@ -2955,8 +2962,14 @@ inline float plan_cost_us(int64_t M, int64_t N, int64_t K, int config, int split
   // has to take in beside its rows of B shrinks with them: 64 x 28672 x 8192 unsplit 42.4 us = 6.3 MB/us)
   const float rows_a = (float)M / (float)((M + c.bm - 1) / c.bm);
   // (not below 33 rows: there the estimate would undercut the streaming kernels, which measure 25 % ahead)
-  const float fill = (config == 1 || config == kDeepSmallConfig) && M > 32 ? fmaxf(0.75f, (rows_a + (float)c.bn) / (float)(c.bm + c.bn)) : 1.0f;
-  const float stream = ((float)M * (float)K + (float)N * (float)K) * fill / (c.stream_bytes_per_us * policy * busy);
+  // (with short rows, K up to 4096, the allowance holds for any M: there the streaming kernels pay for every workgroup's
+  // start and do not measure ahead, 1 x 128256 x 2048 44.7 us with 128x128 tiles against 50.6)
+  const float fill = (config == 1 || config == kDeepSmallConfig) && (M > 32 || K <= 4096) ? fmaxf(0.75f, (rows_a + (float)c.bn) / (float)(c.bm + c.bn)) : 1.0f;
+  // (the 256-column tiles of one tile row stream less with short rows, where a tile is over after a few steps: of
+  // their rate at K >= 4096 they reach 0.8 up to K = 2048 and 0.87 at 2560; 1 x 128256 x 2048 46.8 us with 64x256
+  // tiles and 49.6 with 128x256, 2 x 115072 x 2560 50.6 and 53.2, 1 x 128256 x 4096 79.5 and 81.7)
+  const float short_rows = (config == 3 || config == 4) && K < 4096 ? fmaxf(0.8f, 0.8f + 0.2f * (float)(K - 2048) / 2048.0f) : 1.0f;
+  const float stream = ((float)M * (float)K + (float)N * (float)K) * fill / (c.stream_bytes_per_us * policy * busy * short_rows);
   if (t < stream) t = stream;
   if (splits > 1) t += 3.0f + 2.0f * (float)splits * (float)M * (float)N * 4.0f / 5.0e6f;
   return t;
