@@ -39,7 +39,9 @@ SHAPES = [(32, 8192, 8192, False), (64, 8192, 8192, False), (128, 8192, 8192, Fa
           (1024, 2048, 4096, False), (2048, 2048, 2048, False), (1024, 1024, 8192, False), (1024, 2048, 16384, False),
           (768, 2048, 2048, False),
           # narrow panels with long rows: a few workgroups that each stream a long tile
-          (1, 2048, 28672, False), (8, 1024, 28672, False), (16, 1024, 16384, False)]
+          (1, 2048, 28672, False), (8, 1024, 28672, False), (16, 1024, 16384, False),
+          # a vocabulary-wide panel with short rows (the output projection of a small model)
+          (1, 128256, 2048, False), (8, 128256, 2048, False)]
 
 
 @pytest.mark.parametrize("m,n,k,bias", SHAPES)
