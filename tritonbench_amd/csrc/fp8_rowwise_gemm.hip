@@ -2940,9 +2940,15 @@ inline float plan_cost_us(int64_t M, int64_t N, int64_t K, int config, int split
   // with 252, 2560 x 8192 x 1024 26.6 with 448 where 128x256 tiles take 30.3; over several rounds the table's 9 us per
   // tile stands: it leaves the estimate as far above the measurement as that of the 256x256 tiles, 3-4 %, and the order
   // of the two right: 896 x 57344 x 8192 343 us with 256x256 tiles, 354 with these)
-  const float us_per_item = config == 5 && items <= 2 * slots ? 7.0f : c.us_per_item;
-  float t = full_rounds * (sps * c.us_per_step * step_scale + us_per_item);
-  if (rest) t += sps * (rest <= kNumCu ? c.us_per_step_alone : c.us_per_step) * step_scale + us_per_item;
+  // (64x256 tiles, unsplit, over very short rows, K up to 1664: the table's constants are those of long weight panels;
+  // here a step takes 0.54 us and a tile 5 beside its steps: 400 x 8704 x 1536 10.8 us with 238 tiles, 3 x 45376 x 1024
+  // 11.6 with 178, 192 x 21312 x 1024 8.9 with 252. Only where 128x128 tiles are more than one round: up to that the
+  // deep 128x128 form measures ahead, 400 x 8192 x 1024 7.7 us against 8.5, and its own estimate is a cautious one.)
+  const bool short_c3 = config == 3 && splits == 1 && K <= 13 * kStepK && ((M + 127) / 128) * ((N + 127) / 128) > kNumCu;
+  const float us_per_item = config == 5 && items <= 2 * slots ? 7.0f : short_c3 ? 5.0f : c.us_per_item;
+  const float us_step = short_c3 ? 0.54f : c.us_per_step, us_step_alone = short_c3 ? 0.54f : c.us_per_step_alone;
+  float t = full_rounds * (sps * us_step * step_scale + us_per_item);
+  if (rest) t += sps * (rest <= kNumCu ? us_step_alone : us_step) * step_scale + us_per_item;
   // (the deep 128x128 form is for one round only; beyond 128 workgroups its steps slow down with the chip's
   // clock and the shared L2: 0.49 us with 128, 0.58 with 256)
   if (config == kDeepSmallConfig) {
