@@ -41,7 +41,7 @@ SHAPES = [(32, 8192, 8192, False), (64, 8192, 8192, False), (128, 8192, 8192, Fa
           # narrow panels with long rows: a few workgroups that each stream a long tile
           (1, 2048, 28672, False), (8, 1024, 28672, False), (16, 1024, 16384, False),
           # a vocabulary-wide panel with short rows (the output projection of a small model)
-          (1, 128256, 2048, False), (8, 128256, 2048, False)]
+          (1, 128256, 2048, False), (8, 128256, 2048, False), (1, 151936, 1536, False)]
 
 
 @pytest.mark.parametrize("m,n,k,bias", SHAPES)

@@ -2945,7 +2945,9 @@ inline float plan_cost_us(int64_t M, int64_t N, int64_t K, int config, int split
   // 11.6 with 178, 192 x 21312 x 1024 8.9 with 252. Only where 128x128 tiles are more than one round: up to that the
   // deep 128x128 form measures ahead, 400 x 8192 x 1024 7.7 us against 8.5, and its own estimate is a cautious one.)
   const bool short_c3 = config == 3 && splits == 1 && K <= 13 * kStepK && ((M + 127) / 128) * ((N + 127) / 128) > kNumCu;
-  const float us_per_item = config == 5 && items <= 2 * slots ? 7.0f : short_c3 ? 5.0f : c.us_per_item;
+  // (128x256 tiles over fewer than 8 steps: what a launch costs before its first step is not in the table's 2.6 us a
+  // tile, 2129 x 32 x 512 7.2 us with 17 tiles where 128x128 tiles take 5.2: such launches are left to those)
+  const float us_per_item = config == 5 && items <= 2 * slots ? 7.0f : short_c3 ? 5.0f : config == 4 && sps < 8 ? 10.0f : c.us_per_item;
   const float us_step = short_c3 ? 0.54f : c.us_per_step, us_step_alone = short_c3 ? 0.54f : c.us_per_step_alone;
   float t = full_rounds * (sps * us_step * step_scale + us_per_item);
   if (rest) t += sps * (rest <= kNumCu ? us_step_alone : us_step) * step_scale + us_per_item;
