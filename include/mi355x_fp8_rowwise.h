@@ -234,7 +234,7 @@ int mi355x_fp8_rowwise_gemm_noalloc(const void* a, const void* b,
  * The sizes are read by the kernel, not by the host (no synchronisation): negative sizes
  * count as 0 and rows past M are cut off, so the kernel never leaves A or C whatever the
  * sizes say. Rows of C past the sum of the sizes are left untouched. `tile_config` is -1
- * (the library picks from M / G) or one of the tile configurations listed above.
+ * (the library picks from M / G and the tile counts) or one of the first three tile configurations listed above.
  * Same alignment requirements as mi355x_fp8_rowwise_gemm.
  */
 int mi355x_fp8_rowwise_grouped_gemm(const void* a, const void* b,

@@ -3617,8 +3617,15 @@ int mi355x_fp8_rowwise_grouped_gemm(const void* a, const void* b, const float* a
   hipStream_t s = (hipStream_t)stream;
   // Large tiles when an average group fills most of one and there are enough of them for every
   // CU, small tiles otherwise (the group sizes themselves are on the device; M / G is what the
-  // host knows).
-  if (tile_config < 0) tile_config = (M / G >= 192 && (M / 256) * (N / 256) >= 192) ? 0 : 1;
+  // host knows). Where 256x256 tiles are too few and 256x128 tiles come to about one round of workgroups,
+  // those, on rows long enough for their deeper ring to pay (measured, equal groups: G = 4, M = 1024,
+  // N = K = 8192 78.8 -> 60.9 us; G = 2 ... 16, M = 4096, N = 2048, K = 7168 52-65 -> 49-60; at K = 2048
+  // they are 1-3 % behind the small tiles).
+  if (tile_config < 0) {
+    const bool rows_fill = M / G >= 192;
+    const int64_t tiles_256 = (M / 256) * (N / 256), tiles_128 = (M / 256) * (N / 128);
+    tile_config = rows_fill && tiles_256 >= 192 ? 0 : rows_fill && tiles_128 >= 192 && tiles_128 <= 288 && K >= 4096 ? 2 : 1;
+  }
   const bool ktail = K % kStepK;
   if (tile_config == 0)
     return ktail ? launch_tiled<256, 256, 2, 2, true, kEpiPlain, true>(p, s)
