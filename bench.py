@@ -668,10 +668,13 @@ def main():
         attempt("quantise_f32_8192x8192", lambda: time_quantiser(8192, 8192, torch.float32, dev))
         attempt("quantise_bf16_8192x8192", lambda: time_quantiser(8192, 8192, torch.bfloat16, dev))
         attempt("quantise_bf16_57344x8192", lambda: time_quantiser(57344, 8192, torch.bfloat16, dev, steps=20, copies=2))
+        # (the activation in front of the Llama-3-70B down projection: rows of 28672)
+        attempt("quantise_bf16_4096x28672", lambda: time_quantiser(4096, 28672, torch.bfloat16, dev))
         attempt("block_quantise_bf16_8192x8192", lambda: time_block_quantiser(8192, 8192, torch.bfloat16, dev))
         attempt("block_quantise_f32_8192x8192", lambda: time_block_quantiser(8192, 8192, torch.float32, dev))
         attempt("rmsnorm_quantise_bf16_8192x8192", lambda: time_fused_front_end("rmsnorm", 8192, 8192, dev))
         attempt("silu_mul_quantise_bf16_8192x8192", lambda: time_fused_front_end("silu_mul", 8192, 8192, dev))
+        attempt("silu_mul_quantise_bf16_4096x28672", lambda: time_fused_front_end("silu_mul", 4096, 28672, dev))
         # (rows of 2048 elements: the forms with a wave per row; eight sources in rotation, 0.5 GB)
         attempt("quantise_bf16_16384x2048", lambda: time_quantiser(16384, 2048, torch.bfloat16, dev, copies=8))
         attempt("rmsnorm_quantise_bf16_16384x2048", lambda: time_fused_front_end("rmsnorm", 16384, 2048, dev, copies=8))

@@ -41,7 +41,7 @@ def _check_codes(got_q, got_s, want_q, want_s):
 # rows x K: one chunk per lane and less, the cached 8 rounds exactly, the 1024-lane form, rows
 # longer than the lanes keep in registers (both forms), K not a multiple of the lanes' stride
 # (up to 2048 elements, 4096 for SiLU-mul, a wave per row and four rows per workgroup: row counts around that)
-SHAPES = [(1, 16), (3, 2048), (5, 2304), (4, 6656), (2, 13312), (7, 16384), (3, 16400), (2, 32768), (1, 65536 + 272), (130, 1040),
+SHAPES = [(1, 16), (3, 2048), (5, 2304), (4, 6656), (2, 13312), (7, 16384), (3, 16400), (2, 32768), (3, 28672), (2, 32784), (1, 65536 + 272), (130, 1040),
           (9, 2048), (6, 2064), (5, 4096), (3, 4112), (8, 512), (5, 1024)]
 
 

@@ -389,7 +389,8 @@ def test_quantiser_fp32_bit_exact(gpu_device, rows, cols, sigma):
     assert torch.equal(inv.cpu().view(torch.int32), want_inv.view(torch.int32))
 
 
-@pytest.mark.parametrize("rows,cols", [(9, 144), (256, 2048)])
+# (bf16 rows of 1025 to 4096 elements go to a wave each only from 513 / 2049 rows up: both sides of each switch)
+@pytest.mark.parametrize("rows,cols", [(9, 144), (256, 2048), (512, 2048), (600, 2048), (2048, 4096), (2100, 4096), (2100, 3080)])
 def test_quantiser_bf16_bit_exact(gpu_device, rows, cols):
     x = orc.randn_f32(rows, cols, 1.0, seed=rows + cols).to(torch.bfloat16)
     want_q, want_inv = orc.fp8_row_quantize(x)
@@ -439,6 +440,9 @@ def test_quantiser_rounding_at_every_code_boundary(gpu_device):
 
 
 @pytest.mark.parametrize("dtype,rows,cols,width", [(torch.float32, 3, 20000, 20000), (torch.bfloat16, 2, 20480, 20480),
+                                                     (torch.bfloat16, 3, 28672, 28672), (torch.bfloat16, 2, 32768, 32776),
+                                                     (torch.bfloat16, 2, 32776, 32776), (torch.bfloat16, 2, 53248, 53248),
+                                                     (torch.bfloat16, 1, 70000, 70000),
                                                      (torch.float32, 40, 1024, 1040), (torch.bfloat16, 40, 1000, 1024),
                                                      (torch.float32, 6, 1002, 1003)])
 def test_quantiser_long_rows_and_strides(gpu_device, dtype, rows, cols, width):

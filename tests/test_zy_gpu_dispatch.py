@@ -5,9 +5,13 @@ clearly slower than one of its alternatives. Needs an MI355X.
 
 Timing (tritonbench_amd/tuning.py, the module behind the autotuned backend): a captured graph of
 16 launches over rotating operand sets (cold weights, as a model's are), sustained bursts, the
-median of three. The bar is 15 %: repeated measurements of one and the same plan on the shorter of
+median of three. The bar is 25 %: repeated measurements of one and the same plan on the shorter of
 these shapes (10-30 us) differ by up to 8 % within a run (1 x 8192 x 16384 and 2048^3 have both shown
-the automatic choice and the identical pinned plan that far apart).
+the automatic choice and the identical pinned plan that far apart), and plans of two launches move
+more than that from run to run: 1024 x 1024 x 8192 in four splits has measured 19.7 to 26.8 us over
+eight runs (its second kernel alone 4.9 to 7.1) with the unsplit plans beside it steady to 0.1 us.
+A table that has drifted shows well beyond the bar (the 128x256 constants once put nineteen small
+shapes 30-45 % off).
 
 These are wall-clock assertions, not parity: they carry the `perf` marker beside `gpu`
 (`-m "gpu and not perf"` leaves them out), every shape prints its margin, and the file sorts behind
@@ -19,7 +23,7 @@ from tritonbench_amd import _lib, tuning
 
 pytestmark = [pytest.mark.gpu, pytest.mark.perf]
 
-TOLERANCE = 1.15
+TOLERANCE = 1.25
 # decode- and small-prefill-sized rows of the Llama-3-70B projection sweep, and the small ragged shape with bias
 SHAPES = [(32, 8192, 8192, False), (64, 8192, 8192, False), (128, 8192, 8192, False), (128, 10240, 8192, False),
           (32, 10240, 8192, False), (256, 8192, 8192, False), (1000, 3000, 4112, True),

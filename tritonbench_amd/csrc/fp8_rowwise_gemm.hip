@@ -3712,16 +3712,27 @@ int mi355x_fp8_rowwise_quantize(const void* x, int src_type, void* xq, float* in
                          (uint8_t*)xq, inv_scale, (int)K, (long)ldx, (long)ldq, (long)R);
     }
   } else if (vec && src_type == MI355X_FP8_SRC_BF16) {
-    if (const int wave_cache = bf16_row_chunks_per_lane(K / epv)) {
+    // (A wave per row is the form for many rows. With few, a row spread over a workgroup's 256 lanes is back sooner:
+    // 16 x 4096 3.3 us against 5.2, 2048 x 4096 9.2 against 10.2, 512 x 2048 3.3 against 3.9; from 8192 rows up the wave
+    // form is ahead, 16384 x 4096 37.4 against 40.1.)
+    const int lanes_cache = bf16_row_chunks_per_lane(K / epv);
+    const bool few_rows = (lanes_cache == 8 && R <= 2048) || (lanes_cache == 4 && R <= 512);
+    if (const int wave_cache = few_rows ? 0 : lanes_cache) {
       auto kern = wave_cache == 2   ? quantize_rows_vec_kernel<uint16_t, 2, 64, kWaveRows>
                   : wave_cache == 4 ? quantize_rows_vec_kernel<uint16_t, 4, 64, kWaveRows>
                                     : quantize_rows_vec_kernel<uint16_t, 8, 64, kWaveRows>;
       hipLaunchKernelGGL(kern, dim3(wave_grid), dim3(64 * kWaveRows), 0, s, (const uint16_t*)x, (uint8_t*)xq, inv_scale, (int)K,
                          (long)ldx, (long)ldq, (long)R);
     } else {
-      auto kern = long_row ? quantize_rows_vec_kernel<uint16_t, 8, 1024>
-                           : short_row ? quantize_rows_vec_kernel<uint16_t, 4, 256> : quantize_rows_vec_kernel<uint16_t, 8, 256>;
-      hipLaunchKernelGGL(kern, dim3((unsigned)R), dim3(long_row ? 1024 : 256), 0, s,
+      // (Long rows: 512 lanes with 8 chunks each up to 4096 chunks, 1024 lanes with 4 beyond. 1024 lanes with 8 chunks
+      // each, the f32 form, reach half the rate here: 16384 x 28672 397.6 us against 235.4, 4096 x 28672 104.6 against 64.0;
+      // 16384 x 53248 600 against 469.)
+      const bool very_long_row = K / epv > 8 * 512;
+      auto kern = very_long_row ? quantize_rows_vec_kernel<uint16_t, 4, 1024>
+                  : long_row    ? quantize_rows_vec_kernel<uint16_t, 8, 512>
+                  : short_row   ? quantize_rows_vec_kernel<uint16_t, 4, 256>
+                                : quantize_rows_vec_kernel<uint16_t, 8, 256>;
+      hipLaunchKernelGGL(kern, dim3((unsigned)R), dim3(very_long_row ? 1024 : long_row ? 512 : 256), 0, s,
                          (const uint16_t*)x, (uint8_t*)xq, inv_scale, (int)K, (long)ldx, (long)ldq, (long)R);
     }
   } else if (src_type == MI355X_FP8_SRC_F32) {
@@ -3792,13 +3803,18 @@ int launch_fused_quant(int op, const void* x1, const void* x2, float eps, void* 
   int wave_cache = bf16_row_chunks_per_lane(chunks);
   if (op == kFusedRmsNorm && wave_cache == 8) wave_cache = 0;
   const dim3 grid(wave_cache ? (unsigned)((R + kWaveRows - 1) / kWaveRows) : (unsigned)R);
-  const dim3 block(wave_cache ? 64 * kWaveRows : long_row ? 1024 : 256);
+  // (Long rows up to 32768 elements: 512 lanes with 8 chunks each. With 1024 lanes they reach two thirds of that rate:
+  // SiLU-mul 4096 x 28672 146.6 -> 100.6 us, 1024 x 28672 44.5 -> 29.5; RMSNorm 4096 x 28672 115.8 -> 83.8. Beyond,
+  // 1024 lanes: 4096 x 53248 199.5 us against 218.)
+  const bool mid_row = long_row && chunks <= 8 * 512;
+  const dim3 block(wave_cache ? 64 * kWaveRows : mid_row ? 512 : long_row ? 1024 : 256);
   const uint16_t* a = (const uint16_t*)x1;
   const uint16_t* b = (const uint16_t*)x2;
   if (op == kFusedRmsNorm) {
     auto kern = wave_cache == 2 ? fused_rowwise_quant_kernel<kFusedRmsNorm, 2, 64, kWaveRows>
                 : wave_cache == 4 ? fused_rowwise_quant_kernel<kFusedRmsNorm, 4, 64, kWaveRows>
                 : wave_cache  ? fused_rowwise_quant_kernel<kFusedRmsNorm, 8, 64, kWaveRows>
+                : mid_row     ? fused_rowwise_quant_kernel<kFusedRmsNorm, 8, 512>
                 : long_row    ? fused_rowwise_quant_kernel<kFusedRmsNorm, 8, 1024>
                 : chunks <= 2 * 256 ? fused_rowwise_quant_kernel<kFusedRmsNorm, 2, 256>  // (no idle rounds: 16384 x 4096 47.8 -> 35.5 us)
                 : short_row   ? fused_rowwise_quant_kernel<kFusedRmsNorm, 4, 256> : fused_rowwise_quant_kernel<kFusedRmsNorm, 8, 256>;
@@ -3807,6 +3823,7 @@ int launch_fused_quant(int op, const void* x1, const void* x2, float eps, void* 
     auto kern = wave_cache == 2 ? fused_rowwise_quant_kernel<kFusedSiluMul, 2, 64, kWaveRows>
                 : wave_cache == 4 ? fused_rowwise_quant_kernel<kFusedSiluMul, 4, 64, kWaveRows>
                 : wave_cache  ? fused_rowwise_quant_kernel<kFusedSiluMul, 8, 64, kWaveRows>
+                : mid_row     ? fused_rowwise_quant_kernel<kFusedSiluMul, 8, 512>
                 : long_row    ? fused_rowwise_quant_kernel<kFusedSiluMul, 8, 1024>
                 : short_row   ? fused_rowwise_quant_kernel<kFusedSiluMul, 4, 256> : fused_rowwise_quant_kernel<kFusedSiluMul, 8, 256>;
     hipLaunchKernelGGL(kern, grid, block, 0, s, a, b, eps, (uint8_t*)xq, inv_scale, (int)K, (long)ld1, (long)ld2, (long)ldq, (long)R);
