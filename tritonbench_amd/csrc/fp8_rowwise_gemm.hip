@@ -2534,8 +2534,9 @@ __global__ __launch_bounds__(THREADS* ROWS) void fused_rowwise_quant_kernel(cons
   auto silu_mul = [](float a, float b) -> float { return (a * __builtin_amdgcn_rcpf(1.0f + __expf(-a))) * b; };
 
   float vals[CACHE][EPV];
-  // (the 1024-lane form has 128 registers per lane and none to spare for them)
-  constexpr bool EARLY_WEIGHTS = OP == kFusedRmsNorm && THREADS <= 256;
+  // (the 1024-lane form has 128 registers per lane and none to spare for them; with 512 lanes and 8 chunks each the
+  // weights' registers cost more than the second trip: 8192 x 28672 245 us with them, 167 without)
+  constexpr bool EARLY_WEIGHTS = OP == kFusedRmsNorm && (THREADS <= 256 || (THREADS == 512 && CACHE <= 4));
   v4i wts[EARLY_WEIGHTS ? CACHE : 1];
   float rstd = 0.0f;
   if (OP == kFusedRmsNorm) {
@@ -3807,7 +3808,11 @@ int launch_fused_quant(int op, const void* x1, const void* x2, float eps, void* 
   // SiLU-mul 4096 x 28672 146.6 -> 100.6 us, 1024 x 28672 44.5 -> 29.5; RMSNorm 4096 x 28672 115.8 -> 83.8. Beyond,
   // 1024 lanes: 4096 x 53248 199.5 us against 218.)
   const bool mid_row = long_row && chunks <= 8 * 512;
-  const dim3 block(wave_cache ? 64 * kWaveRows : mid_row ? 512 : long_row ? 1024 : 256);
+  // (Rows of 8193 to 16384 elements: 512 lanes with 4 chunks each instead of 256 with 8. RMSNorm 8192 x 16384 96.0 ->
+  // 78.6 us, 32768 x 16384 370 -> 302, 8192 x 11008 85.1 -> 67.1; SiLU-mul 8192 x 11008 80.6 -> 79.6, 8192 x 16384
+  // 109.1 -> 107.6.)
+  const bool half_row = !wave_cache && !long_row && !short_row;
+  const dim3 block(wave_cache ? 64 * kWaveRows : mid_row || half_row ? 512 : long_row ? 1024 : 256);
   const uint16_t* a = (const uint16_t*)x1;
   const uint16_t* b = (const uint16_t*)x2;
   if (op == kFusedRmsNorm) {
@@ -3817,7 +3822,7 @@ int launch_fused_quant(int op, const void* x1, const void* x2, float eps, void* 
                 : mid_row     ? fused_rowwise_quant_kernel<kFusedRmsNorm, 8, 512>
                 : long_row    ? fused_rowwise_quant_kernel<kFusedRmsNorm, 8, 1024>
                 : chunks <= 2 * 256 ? fused_rowwise_quant_kernel<kFusedRmsNorm, 2, 256>  // (no idle rounds: 16384 x 4096 47.8 -> 35.5 us)
-                : short_row   ? fused_rowwise_quant_kernel<kFusedRmsNorm, 4, 256> : fused_rowwise_quant_kernel<kFusedRmsNorm, 8, 256>;
+                : short_row   ? fused_rowwise_quant_kernel<kFusedRmsNorm, 4, 256> : fused_rowwise_quant_kernel<kFusedRmsNorm, 4, 512>;
     hipLaunchKernelGGL(kern, grid, block, 0, s, a, b, eps, (uint8_t*)xq, inv_scale, (int)K, (long)ld1, (long)ld2, (long)ldq, (long)R);
   } else {
     auto kern = wave_cache == 2 ? fused_rowwise_quant_kernel<kFusedSiluMul, 2, 64, kWaveRows>
@@ -3825,7 +3830,7 @@ int launch_fused_quant(int op, const void* x1, const void* x2, float eps, void* 
                 : wave_cache  ? fused_rowwise_quant_kernel<kFusedSiluMul, 8, 64, kWaveRows>
                 : mid_row     ? fused_rowwise_quant_kernel<kFusedSiluMul, 8, 512>
                 : long_row    ? fused_rowwise_quant_kernel<kFusedSiluMul, 8, 1024>
-                : short_row   ? fused_rowwise_quant_kernel<kFusedSiluMul, 4, 256> : fused_rowwise_quant_kernel<kFusedSiluMul, 8, 256>;
+                : short_row   ? fused_rowwise_quant_kernel<kFusedSiluMul, 4, 256> : fused_rowwise_quant_kernel<kFusedSiluMul, 4, 512>;
     hipLaunchKernelGGL(kern, grid, block, 0, s, a, b, eps, (uint8_t*)xq, inv_scale, (int)K, (long)ld1, (long)ld2, (long)ldq, (long)R);
   }
   hipError_t e = hipGetLastError();
